@@ -1,0 +1,116 @@
+/*
+ * libquest_hip -- C ABI of the MI355X (gfx950) kernels behind the `quest` Python package.
+ *
+ * Every entry point is what the reference's torch extension binds for the same step: it takes
+ * raw device pointers, plain sizes and the HIP stream to launch on (passed as void*, i.e. a
+ * hipStream_t), borrows every buffer (the caller allocates inputs and outputs), launches
+ * asynchronously and never synchronises or allocates, so calls can be recorded into a HIP
+ * graph.  A NULL optional output means "do not produce it".  The return value is 0 or one of
+ * the negative QUEST_ERR_* codes; nothing is launched when an argument check fails.
+ *
+ * dtype selects the 16-bit float type of activations, scales and outputs.  The reference
+ * instantiates bfloat16 only; float16 is an addition.
+ *
+ * Citations are file:line under gemm-quest/ of the reference.
+ */
+#ifndef QUEST_HIP_H
+#define QUEST_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QUEST_DTYPE_BF16 0
+#define QUEST_DTYPE_FP16 1
+
+#define QUEST_OK 0
+#define QUEST_ERR_NULL_POINTER (-1)  /* a required pointer is NULL */
+#define QUEST_ERR_BAD_SHAPE (-2)     /* size <= 0, odd K, K not a multiple of what the kernel needs */
+#define QUEST_ERR_BAD_DTYPE (-3)     /* dtype is neither QUEST_DTYPE_BF16 nor QUEST_DTYPE_FP16 */
+#define QUEST_ERR_ALIGNMENT (-4)     /* a pointer is not aligned for the vector accesses used */
+#define QUEST_ERR_UNSUPPORTED (-5)   /* shape outside what this build instantiates */
+#define QUEST_ERR_LAUNCH (-6)        /* hipGetLastError() after the launch was not hipSuccess */
+
+/* ABI version of this header (major * 100 + minor). */
+int quest_version(void);
+
+/* Text for a QUEST_ERR_* code (static storage). */
+const char *quest_status_string(int status);
+
+/*
+ * scale[m] = dtype( sqrt(mean_k x[m,k]^2) * fp32(2.513930578568423 * 2 / 15) + 1e-8f ), fp32 inside.
+ * Replaces find_scale_int4_cuda_bf16 (quest/quantize_kernel.cu:97-117; glue quest/quantize.cpp:5-25).
+ * x: (batch_size, group_size) dtype, row-major; scale: (batch_size) dtype.  group_size % 8 == 0.
+ */
+int quest_find_scale_int4(void *scale, const void *x, int group_size, int batch_size, int dtype, void *stream);
+
+/*
+ * q = clamp(floor(f32(x) / f32(scale[m])), -8, 7) and, each optional:
+ *   x_int[m,k] = q (int8);  x_int_packed[m,j] = (q[2j+1] << 4) | (q[2j] & 0xF);
+ *   x_int_row_sum[m] = sum_k q (int32);  if do_dequantize: x[m,k] = dtype(q * s + s * 0.5f) in place.
+ * Replaces quantize_int4_cuda_bf16 (quest/quantize_kernel.cu:232-261; glue quest/quantize.cpp:28-70).
+ * group_size % 8 == 0.
+ */
+int quest_quantize_int4(void *x, const void *scale, int8_t *x_int, uint8_t *x_int_packed,
+                        int32_t *x_int_row_sum, int group_size, int batch_size, int do_dequantize,
+                        int dtype, void *stream);
+
+/*
+ * mat_d[a,b] = dtype( f32(2 * mat_c[a,b] + vec_a_add[a] + vec_b_add[b]) * (0.5f * vec_a_mul[a] * vec_b_mul[b]) ).
+ * Replaces add_mul_vv_cuda_bf16 (quest/quantize_kernel.cu:309-341; glue quest/quantize.cpp:73-105).
+ */
+int quest_add_mul_vv(void *mat_d, const int32_t *vec_a_add, const void *vec_a_mul,
+                     const int32_t *vec_b_add, const void *vec_b_mul, const int32_t *mat_c,
+                     int size_a, int size_b, int dtype, void *stream);
+
+/*
+ * mat_c (size_m, size_n) int32 = A * B^T with A (size_m, size_k/2) and B (size_n, size_k/2) packed
+ * signed INT4, low nibble = even k.  Replaces matmul_int4_int4t_int32_cuda
+ * (quest/matmul_kernel.cu:8-63; glue quest/matmul.cpp:52-66).  size_k % 32 == 0 (the reference's
+ * CUTLASS alignment), any size_m >= 1 and size_n >= 1.  Pointers 16-byte aligned.
+ */
+int quest_matmul_int4_int4t_int32(int32_t *mat_c, const uint8_t *mat_a, const uint8_t *mat_b,
+                                  int size_m, int size_k, int size_n, void *stream);
+
+/*
+ * mat_d (size_m, size_n) dtype = the same GEMM followed, in registers, by the add_mul_vv formula
+ * above with vec_a_* indexed by row and vec_b_* by column (the int32 accumulator is used exactly,
+ * where the reference's functor first rounds it to fp16).  Replaces
+ * fused_matmul_dequantize_int4_int4t_bf16_cuda (quest/fused_matmul_dequantize_kernel.cu:4-57,
+ * include/symmetric/epilogue/thread/linear_combination_dequant.h:122-185; glue
+ * quest/fused_matmul_dequantize.cpp:20-42).
+ */
+int quest_fused_matmul_dequantize_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                             const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                             const void *vec_a_mul, const void *vec_b_mul,
+                                             int size_m, int size_k, int size_n, int dtype, void *stream);
+
+/*
+ * y = block-128 Walsh-Hadamard transform of every row of x along K, fp32 butterflies, * had_scale,
+ * one rounding to dtype.  had_scale = 181/2048 reproduces F.linear(x.view(-1,128), HADAMARD_MATRIX)
+ * (benchmarks/utils.py:17,89-90: the matrix entries are bf16(2^-3.5) = 181/2048); had_scale = 2^-3.5
+ * reproduces the weight-side hadamard_transform(..., scale=2**-3.5) (benchmarks/utils.py:38-39).
+ * y may alias x.  group_size % 128 == 0.
+ */
+int quest_hadamard128(void *y, const void *x, int group_size, int batch_size, float had_scale,
+                      int dtype, void *stream);
+
+/*
+ * One pass over x that does what linear_forward does before its GEMM (benchmarks/utils.py:89-100):
+ * Hadamard (as quest_hadamard128, optional: had_scale == 0 skips it), scale (as
+ * quest_find_scale_int4 on the transformed row), INT4 codes packed (as quest_quantize_int4) and
+ * their row sums.  x is read once and never written.  x_had, when not NULL, receives the
+ * transformed activations (dtype) the scale and codes were computed from.  scale is required;
+ * x_int_packed and x_int_row_sum are optional.  group_size % 128 == 0, group_size <= 65536.
+ */
+int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t *x_int_packed,
+                                 int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size,
+                                 float had_scale, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QUEST_HIP_H */

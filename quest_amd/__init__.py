@@ -1,0 +1,23 @@
+"""quest_amd: the W4A4 linear-layer inference path of QuEST (gemm-quest) on MI355X / gfx950.
+
+`import quest_amd as quest` gives the reference's `quest` call surface; `quest_amd.harness` holds
+the counterparts of gemm-quest/benchmarks/utils.py (linear_forward, preprocess_weight, Linear4bit,
+the timing helpers).
+"""
+from .api import (  # noqa: F401
+    HADAMARD_ENTRY,
+    add_mul_vv,
+    find_scale_int4,
+    fused_matmul_dequantize_int4_int4t,
+    fused_matmul_dequantize_int4_int4t_bf16,
+    generate_random_meta48_int4,
+    hadamard128,
+    hadamard_quantize_int4,
+    matmul_int4_int4t_int32,
+    matmul_int4sp_int4t_int32,
+    quantize_int4,
+    reorder_meta48_int4,
+    uncompress_meta48_int4,
+)
+
+__version__ = '0.1.0'

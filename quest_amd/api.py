@@ -1,0 +1,195 @@
+"""The `quest` call surface of the reference (gemm-quest/quest/__init__.py:6-130) on MI355X.
+
+Same names, argument order, defaults and return values; the work is done by hand-written HIP
+kernels reached through the C ABI of libquest_hip.so.  Differences, all additive:
+  * float16 is accepted wherever the reference asserts bfloat16;
+  * `hadamard128` and `hadamard_quantize_int4` are new (the fused activation kernel);
+  * the 4:8-sparse entry points raise NotImplementedError (NVIDIA sparse tensor cores only).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import DTYPE_CODE, check, ptr, require_gpu, stream_of
+
+_FLOAT16S = (torch.bfloat16, torch.float16)
+HADAMARD_ENTRY = 181. / 2048.        # bf16(2**-3.5) == fp16(2**-3.5): what the reference's matrix holds
+
+
+def fused_matmul_dequantize_int4_int4t_bf16(
+        mat_a: torch.Tensor,
+        mat_b: torch.Tensor,
+        vec_a_add: torch.Tensor,
+        vec_b_add: torch.Tensor,
+        vec_a_mul: torch.Tensor,
+        vec_b_mul: torch.Tensor,
+        out: torch.Tensor = None,
+) -> torch.Tensor:
+    """gemm-quest/quest/__init__.py:6-20.  The output dtype follows vec_a_mul (bf16 or fp16)."""
+    if out is None:
+        out = torch.empty(mat_a.size(0), mat_b.size(0), dtype=vec_a_mul.dtype, device=mat_a.device)
+    assert mat_a.dtype == torch.uint8 and mat_b.dtype == torch.uint8 and vec_a_add.dtype == torch.int32 and vec_b_add.dtype == torch.int32
+    assert vec_a_mul.dtype in _FLOAT16S and vec_b_mul.dtype == vec_a_mul.dtype and out.dtype == vec_a_mul.dtype
+    assert mat_a.is_contiguous() and mat_b.is_contiguous() and vec_a_add.is_contiguous() and vec_b_add.is_contiguous() and vec_a_mul.is_contiguous() and vec_b_mul.is_contiguous() and out.is_contiguous()
+    assert mat_a.size(1) == mat_b.size(1) and vec_a_add.numel() == mat_a.size(0) and vec_a_mul.numel() == mat_a.size(0)
+    assert vec_b_add.numel() == mat_b.size(0) and vec_b_mul.numel() == mat_b.size(0)
+    assert out.size(0) == mat_a.size(0) and out.size(1) == mat_b.size(0)
+    dev = require_gpu(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, out)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_fused_matmul_dequantize_int4_int4t(
+            ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
+            mat_a.size(0), mat_b.size(1) * 2, mat_b.size(0), DTYPE_CODE[out.dtype], stream_of(out)),
+            'fused_matmul_dequantize_int4_int4t')
+    return out
+
+
+# the same kernel serves both 16-bit float types
+fused_matmul_dequantize_int4_int4t = fused_matmul_dequantize_int4_int4t_bf16
+
+
+def matmul_int4_int4t_int32(
+        mat_a: torch.Tensor,
+        mat_b: torch.Tensor,
+        out: torch.Tensor = None,
+) -> torch.Tensor:
+    """gemm-quest/quest/__init__.py:23-33."""
+    if out is None:
+        out = torch.empty(mat_a.size(0), mat_b.size(0), dtype=torch.int32, device=mat_a.device)
+    assert mat_a.dtype == torch.uint8 and mat_b.dtype == torch.uint8 and out.dtype == torch.int32
+    assert mat_a.is_contiguous() and mat_b.is_contiguous() and out.is_contiguous()
+    assert mat_a.size(1) == mat_b.size(1) and out.size(0) == mat_a.size(0) and out.size(1) == mat_b.size(0)
+    dev = require_gpu(mat_a, mat_b, out)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_matmul_int4_int4t_int32(
+            ptr(out), ptr(mat_a), ptr(mat_b), mat_a.size(0), mat_b.size(1) * 2, mat_b.size(0), stream_of(out)),
+            'matmul_int4_int4t_int32')
+    return out
+
+
+def _sparse_unsupported(*_args, **_kwargs):
+    raise NotImplementedError(
+        'the 4:8-sparse INT4 path of the reference targets NVIDIA sparse tensor cores and is not part of this build')
+
+
+# gemm-quest/quest/__init__.py:36-84
+matmul_int4sp_int4t_int32 = _sparse_unsupported
+reorder_meta48_int4 = _sparse_unsupported
+uncompress_meta48_int4 = _sparse_unsupported
+generate_random_meta48_int4 = _sparse_unsupported
+
+
+def find_scale_int4(
+        x: torch.Tensor,
+        scale: torch.Tensor = None,
+) -> torch.Tensor:
+    """gemm-quest/quest/__init__.py:87-96."""
+    if scale is None:
+        scale = torch.empty(x.size(0), 1, dtype=x.dtype, device=x.device)
+    assert x.dtype in _FLOAT16S and scale.dtype == x.dtype
+    assert x.is_contiguous() and scale.is_contiguous()
+    assert x.dim() == 2 and scale.numel() == x.size(0)
+    dev = require_gpu(x, scale)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_find_scale_int4(ptr(scale), ptr(x), x.size(1), x.size(0), DTYPE_CODE[x.dtype],
+                                                stream_of(x)), 'find_scale_int4')
+    return scale
+
+
+def quantize_int4(
+        x: torch.Tensor,
+        scale: torch.Tensor,
+        x_int: torch.Tensor = None,
+        x_int_packed: torch.Tensor = None,
+        x_int_row_sum: torch.Tensor = None,
+        do_dequantize: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None, torch.Tensor | None]:
+    """gemm-quest/quest/__init__.py:99-114.  Outputs passed as None are not produced."""
+    assert x.dtype in _FLOAT16S and scale.dtype == x.dtype
+    assert x_int is None or x_int.dtype == torch.int8
+    assert x_int_packed is None or x_int_packed.dtype == torch.uint8
+    assert x_int_row_sum is None or x_int_row_sum.dtype == torch.int32
+    assert x.is_contiguous() and scale.is_contiguous()
+    assert all(t is None or t.is_contiguous() for t in (x_int, x_int_packed, x_int_row_sum))
+    assert x.dim() == 2 and scale.numel() == x.size(0)
+    assert x_int is None or x_int.shape == x.shape
+    assert x_int_packed is None or (x_int_packed.size(0) == x.size(0) and x_int_packed.size(1) * 2 == x.size(1))
+    assert x_int_row_sum is None or x_int_row_sum.numel() == x.size(0)
+    dev = require_gpu(x, scale, x_int, x_int_packed, x_int_row_sum)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_quantize_int4(ptr(x), ptr(scale), ptr(x_int), ptr(x_int_packed), ptr(x_int_row_sum),
+                                              x.size(1), x.size(0), int(bool(do_dequantize)), DTYPE_CODE[x.dtype],
+                                              stream_of(x)), 'quantize_int4')
+    return x, x_int, x_int_packed, x_int_row_sum
+
+
+def add_mul_vv(
+        vec_a_add: torch.Tensor,
+        vec_a_mul: torch.Tensor,
+        vec_b_add: torch.Tensor,
+        vec_b_mul: torch.Tensor,
+        mat_c: torch.Tensor,
+        mat_d: torch.Tensor = None,
+) -> torch.Tensor:
+    """gemm-quest/quest/__init__.py:117-130."""
+    if mat_d is None:
+        mat_d = torch.empty(mat_c.shape, dtype=vec_a_mul.dtype, device=mat_c.device)
+    assert vec_a_add.dtype == torch.int32 and vec_b_add.dtype == torch.int32 and mat_c.dtype == torch.int32
+    assert vec_a_mul.dtype in _FLOAT16S and vec_b_mul.dtype == vec_a_mul.dtype and mat_d.dtype == vec_a_mul.dtype
+    assert vec_a_add.is_contiguous() and vec_a_mul.is_contiguous() and vec_b_add.is_contiguous() and vec_b_mul.is_contiguous() and mat_c.is_contiguous() and mat_d.is_contiguous()
+    assert mat_c.dim() == 2 and mat_d.shape == mat_c.shape
+    assert vec_a_add.numel() == mat_c.size(0) and vec_a_mul.numel() == mat_c.size(0)
+    assert vec_b_add.numel() == mat_c.size(1) and vec_b_mul.numel() == mat_c.size(1)
+    dev = require_gpu(vec_a_add, vec_a_mul, vec_b_add, vec_b_mul, mat_c, mat_d)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_add_mul_vv(ptr(mat_d), ptr(vec_a_add), ptr(vec_a_mul), ptr(vec_b_add), ptr(vec_b_mul),
+                                           ptr(mat_c), mat_c.size(0), mat_c.size(1), DTYPE_CODE[mat_d.dtype],
+                                           stream_of(mat_d)), 'add_mul_vv')
+    return mat_d
+
+
+def hadamard128(x: torch.Tensor, out: torch.Tensor = None, scale: float = HADAMARD_ENTRY) -> torch.Tensor:
+    """Block-128 Walsh-Hadamard transform along the last dimension.  scale=181/2048 is the
+    activation transform of linear_forward (gemm-quest/benchmarks/utils.py:17,89-90),
+    scale=2**-3.5 the weight transform of preprocess_weight (utils.py:38-39).  out may be x."""
+    if out is None:
+        out = torch.empty_like(x)
+    assert x.dtype in _FLOAT16S and out.dtype == x.dtype and out.shape == x.shape
+    assert x.is_contiguous() and out.is_contiguous()
+    k = x.size(-1)
+    dev = require_gpu(x, out)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_hadamard128(ptr(out), ptr(x), k, x.numel() // k, float(scale), DTYPE_CODE[x.dtype],
+                                            stream_of(x)), 'hadamard128')
+    return out
+
+
+def hadamard_quantize_int4(
+        x: torch.Tensor,
+        scale: torch.Tensor = None,
+        x_int_packed: torch.Tensor = None,
+        x_int_row_sum: torch.Tensor = None,
+        x_had: torch.Tensor = None,
+        hadamard_scale: float = HADAMARD_ENTRY,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One pass over x: block-128 Hadamard (skipped when hadamard_scale == 0), Gaussian-clip scale,
+    INT4 codes packed two per byte, and their row sums -- the three launches of
+    gemm-quest/benchmarks/utils.py:89-100 in one.  x_had, if given, receives the transformed
+    activations the codes were computed from.  Returns (scale, x_int_packed, x_int_row_sum)."""
+    m, k = x.shape
+    if scale is None:
+        scale = torch.empty(m, 1, dtype=x.dtype, device=x.device)
+    if x_int_packed is None:
+        x_int_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=x.device)
+    if x_int_row_sum is None:
+        x_int_row_sum = torch.empty(m, 1, dtype=torch.int32, device=x.device)
+    assert x.dtype in _FLOAT16S and scale.dtype == x.dtype and x_int_packed.dtype == torch.uint8 and x_int_row_sum.dtype == torch.int32
+    assert x.is_contiguous() and scale.is_contiguous() and x_int_packed.is_contiguous() and x_int_row_sum.is_contiguous()
+    assert scale.numel() == m and x_int_row_sum.numel() == m and x_int_packed.shape == (m, k // 2)
+    assert x_had is None or (x_had.dtype == x.dtype and x_had.shape == x.shape and x_had.is_contiguous())
+    dev = require_gpu(x, scale, x_int_packed, x_int_row_sum, x_had)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_hadamard_quantize_int4(ptr(x), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum),
+                                                       ptr(x_had), k, m, float(hadamard_scale), DTYPE_CODE[x.dtype],
+                                                       stream_of(x)), 'hadamard_quantize_int4')
+    return scale, x_int_packed, x_int_row_sum

@@ -1,0 +1,142 @@
+// Shared device helpers for the gfx950 kernels of libquest_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/quest_hip.h"
+
+namespace quest {
+
+// ---- 16-bit float <-> fp32 ------------------------------------------------------------------
+// DT = QUEST_DTYPE_BF16 (0) or QUEST_DTYPE_FP16 (1); values travel as raw uint16_t bits.
+template <int DT>
+__device__ __forceinline__ float to_f32(uint32_t h16) {
+    if constexpr (DT == QUEST_DTYPE_BF16) {
+        return __uint_as_float(h16 << 16);
+    } else {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)h16);
+    }
+}
+
+// low / high half of a dword holding two 16-bit floats
+template <int DT>
+__device__ __forceinline__ float lo_f32(uint32_t w) {
+    if constexpr (DT == QUEST_DTYPE_BF16) return __uint_as_float(w << 16);
+    else return to_f32<DT>(w & 0xffffu);
+}
+template <int DT>
+__device__ __forceinline__ float hi_f32(uint32_t w) {
+    if constexpr (DT == QUEST_DTYPE_BF16) return __uint_as_float(w & 0xffff0000u);
+    else return to_f32<DT>(w >> 16);
+}
+
+// Round an fp32 value to nearest even.  The empty asm pins `f` as an fp32 register first: without
+// it the compiler folds a preceding fp32 multiply into v_fma_mixlo_f16, which rounds the exact
+// product once to fp16 instead of first to fp32 and then to fp16 as the reference arithmetic does.
+template <int DT>
+__device__ __forceinline__ uint32_t from_f32(float f) {
+    asm volatile("" : "+v"(f));
+    if constexpr (DT == QUEST_DTYPE_BF16) {
+        return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+    } else {
+        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+}
+template <int DT>
+__device__ __forceinline__ uint32_t pack2_from_f32(float lo, float hi) {
+    return from_f32<DT>(lo) | (from_f32<DT>(hi) << 16);
+}
+
+// ---- cross-lane moves -----------------------------------------------------------------------
+// value of lane (lane ^ M); M = 1, 2, 8 are single DPP moves, 4 and 16 LDS-crossbar swizzles.
+template <int M>
+__device__ __forceinline__ int lane_xor_i(int v) {
+    if constexpr (M == 1) return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);        // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    else if constexpr (M == 4) return __builtin_amdgcn_ds_swizzle(v, (4 << 10) | 0x1F);
+    else if constexpr (M == 8) return __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true);  // row_ror:8
+    else if constexpr (M == 16) return __builtin_amdgcn_ds_swizzle(v, (16 << 10) | 0x1F);
+    else return __shfl_xor(v, 32, 64);
+}
+template <int M>
+__device__ __forceinline__ float lane_xor_f(float v) {
+    return __int_as_float(lane_xor_i<M>(__float_as_int(v)));
+}
+
+// Butterfly all-reduce over the 64 lanes; every lane ends with the same bits (fixed order).
+__device__ __forceinline__ float wave_sum_f(float v) {
+    v += lane_xor_f<1>(v);
+    v += lane_xor_f<2>(v);
+    v += lane_xor_f<4>(v);
+    v += lane_xor_f<8>(v);
+    v += lane_xor_f<16>(v);
+    v += lane_xor_f<32>(v);
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+    v += lane_xor_i<1>(v);
+    v += lane_xor_i<2>(v);
+    v += lane_xor_i<4>(v);
+    v += lane_xor_i<8>(v);
+    v += lane_xor_i<16>(v);
+    v += lane_xor_i<32>(v);
+    return v;
+}
+
+// Block all-reduce through LDS: per-wave totals are added in wave order by every thread.
+// `slots` must hold BLOCK / 64 entries; two barriers, so it can be reused right after.
+template <int BLOCK>
+__device__ __forceinline__ float block_sum_f(float v, float *slots) {
+    v = wave_sum_f(v);
+    if constexpr (BLOCK == 64) return v;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    float t = slots[0];
+#pragma unroll
+    for (int w = 1; w < BLOCK / 64; w++) t += slots[w];
+    __syncthreads();
+    return t;
+}
+template <int BLOCK>
+__device__ __forceinline__ int block_sum_i(int v, int *slots) {
+    v = wave_sum_i(v);
+    if constexpr (BLOCK == 64) return v;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    int t = slots[0];
+#pragma unroll
+    for (int w = 1; w < BLOCK / 64; w++) t += slots[w];
+    __syncthreads();
+    return t;
+}
+
+// ---- the quantiser ---------------------------------------------------------------------------
+// fp32(2.513930578568423 * 2 / 15): the Gaussian-MSE-optimal INT4 clip over 7.5 steps.
+__device__ constexpr float kGaussInt4Step = 0.3351907438091231f;
+__device__ constexpr float kScaleEps = 1e-8f;
+
+// scale from a row's sum of squares; separate multiply and add (no fused multiply-add), as the
+// PyTorch statement of the rule evaluates it.
+__device__ __forceinline__ float scale_from_sumsq(float sumsq, int k) {
+    float mean_sq = __fdiv_rn(sumsq, (float)k);
+    float sd = __fsqrt_rn(mean_sq);
+    return __fadd_rn(__fmul_rn(sd, kGaussInt4Step), kScaleEps);
+}
+
+// clamp(floor(x / s), -8, 7) with an IEEE-correct divide; NaN quotients (0/0) land on -8 like
+// fmaxf/fminf in the CUDA kernel this replaces.
+__device__ __forceinline__ float quant_code(float x, float s) {
+    float q = __builtin_floorf(__fdiv_rn(x, s));
+    q = fmaxf(q, -8.f);
+    q = fminf(q, 7.f);
+    return q;
+}
+
+inline int check_dtype(int dtype) { return dtype == QUEST_DTYPE_BF16 || dtype == QUEST_DTYPE_FP16; }
+inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+inline int launch_status() { return hipGetLastError() == hipSuccess ? QUEST_OK : QUEST_ERR_LAUNCH; }
+
+}  // namespace quest

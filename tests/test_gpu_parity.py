@@ -1,0 +1,261 @@
+"""GPU parity: every HIP entry point, called through the C ABI (quest_amd.api -> ctypes ->
+libquest_hip.so), against the CPU oracle on the same seeded inputs.
+
+Bars: INT4 codes, packed bytes, row sums, int32 accumulators and the scale epilogue are bit-exact;
+the Hadamard output agrees with the reference's matmul formulation to <= 1e-3 relative (and is
+bit-identical to the fp32-butterfly statement of the oracle); the per-row scale may differ from a
+torch-CPU reduction by one 16-bit ulp on a rare row (summation order), which is counted and bounded.
+"""
+import pytest
+import torch
+
+from oracle import quest_oracle as qo
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16]
+DEV = 'cuda:0'
+
+
+@pytest.fixture(scope='module')
+def quest():
+    import quest_amd
+    from quest_amd import _lib
+    _lib.load()                       # fails loudly if the HIP library is not built
+    assert torch.cuda.is_available()
+    return quest_amd
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16).to(torch.int32)
+
+
+def ulp_diff(a, b):
+    return (bits(a.cpu()) - bits(b.cpu())).abs()
+
+
+def rand_act(m, k, dtype, seed, spread=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g)
+    if spread:
+        x = x * (torch.rand(m, 1, generator=g) * 4 + 0.05)
+    return x.to(dtype)
+
+
+# --------------------------------------------------------------------------- S1
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 768), (37, 4096), (1, 128), (8, 11008), (3, 16384)])
+def test_find_scale(quest, dtype, shape):
+    x = rand_act(*shape, dtype, seed=1)
+    want = qo.find_scale_int4(x)
+    got = quest.find_scale_int4(x.to(DEV)).cpu()
+    d = ulp_diff(got, want)
+    assert d.max() <= 1, 'scale differs from the oracle by more than one ulp'
+    assert (d != 0).sum() <= max(1, shape[0] // 100), f'{int((d != 0).sum())} rows differ'
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_find_scale_constant_rows_exact(quest, dtype):
+    vals = torch.tensor([0., 1., -1., 0.5, 3., -7.25, 100., 2. ** -10])
+    x = vals.to(dtype)[:, None].repeat(1, 512).contiguous()
+    assert torch.equal(quest.find_scale_int4(x.to(DEV)).cpu(), qo.find_scale_int4(x))
+
+
+# --------------------------------------------------------------------------- S2
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 768), (5, 4096), (1, 8), (16, 11008)])
+def test_quantize_all_outputs_bit_exact(quest, dtype, shape):
+    m, k = shape
+    x = rand_act(m, k, dtype, seed=2)
+    scale = qo.find_scale_int4(x)
+    xi = torch.empty(m, k, dtype=torch.int8)
+    xp = torch.empty(m, k // 2, dtype=torch.uint8)
+    rs = torch.empty(m, 1, dtype=torch.int32)
+    xd = x.clone()
+    qo.quantize_int4(xd, scale, xi, xp, rs, True)
+    gx = x.to(DEV)
+    gi = torch.empty(m, k, dtype=torch.int8, device=DEV)
+    gp = torch.empty(m, k // 2, dtype=torch.uint8, device=DEV)
+    gs = torch.empty(m, 1, dtype=torch.int32, device=DEV)
+    out = quest.quantize_int4(gx, scale.to(DEV), gi, gp, gs, True)
+    assert out[0] is gx and out[1] is gi and out[2] is gp and out[3] is gs
+    assert torch.equal(gi.cpu(), xi)
+    assert torch.equal(gp.cpu(), xp)
+    assert torch.equal(gs.cpu(), rs)
+    assert torch.equal(bits(gx.cpu()), bits(xd))
+    # optional outputs left out: x untouched, only what was asked for is written
+    gx2 = x.to(DEV)
+    gp2 = torch.zeros_like(gp)
+    r = quest.quantize_int4(gx2, scale.to(DEV), None, gp2, None, False)
+    assert r[1] is None and r[3] is None
+    assert torch.equal(gp2.cpu(), xp) and torch.equal(bits(gx2.cpu()), bits(x))
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_quantize_every_16bit_input(quest, dtype):
+    """All 65536 bit patterns as inputs (NaN/Inf rows aside) against a spread of scales."""
+    allbits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    finite = torch.isfinite(allbits.float())
+    vals = torch.where(finite, allbits, torch.zeros_like(allbits))
+    scales = torch.tensor([0.3351907, 1.0, 0.007, 3.1, 2. ** -9, 0.0625, 117.0, 0.99, 0.4062, 5e-4,
+                           0.1234, 0.0101, 12.5, 0.75, 1.5, 2.25]).to(dtype).view(-1, 1)
+    x = vals.view(1, -1).repeat(scales.numel(), 1).contiguous()
+    xi = torch.empty(x.shape, dtype=torch.int8)
+    rs = torch.empty(x.size(0), 1, dtype=torch.int32)
+    qo.quantize_int4(x.clone(), scales, xi, None, rs, False)
+    gi = torch.empty(x.shape, dtype=torch.int8, device=DEV)
+    gs = torch.empty(x.size(0), 1, dtype=torch.int32, device=DEV)
+    quest.quantize_int4(x.to(DEV), scales.to(DEV), gi, None, gs, False)
+    assert torch.equal(gi.cpu(), xi)
+    assert torch.equal(gs.cpu(), rs)
+
+
+# --------------------------------------------------------------------------- E1
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 224), (1, 1), (7, 513), (33, 4096)])
+def test_add_mul_vv(quest, dtype, shape):
+    m, n = shape
+    g = torch.Generator().manual_seed(3)
+    c = torch.randint(-200000, 200000, (m, n), generator=g, dtype=torch.int32)
+    a_add = torch.randint(-30000, 30000, (m, 1), generator=g, dtype=torch.int32)
+    b_add = torch.randint(-30000, 30000, (n, 1), generator=g, dtype=torch.int32)
+    a_mul = (torch.rand(m, 1, generator=g) * 0.09 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype)
+    want = qo.add_mul_vv(a_add, a_mul, b_add, b_mul, c)
+    got = quest.add_mul_vv(a_add.to(DEV), a_mul.to(DEV), b_add.to(DEV), b_mul.to(DEV), c.to(DEV)).cpu()
+    assert torch.equal(bits(got), bits(want))
+
+
+# --------------------------------------------------------------------------- G1 / G2
+def rand_codes(rows, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    return qo.pack_int4(torch.randint(-8, 8, (rows, k), generator=g).to(torch.int8))
+
+
+GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512), (257, 128, 300),
+               (33, 96, 7), (512, 1024, 1024), (300, 160, 257), (256, 2048, 256)]
+
+
+@pytest.mark.parametrize('shape', GEMM_SHAPES)
+def test_matmul_int32_bit_exact(quest, shape):
+    m, k, n = shape
+    a, b = rand_codes(m, k, 4), rand_codes(n, k, 5)
+    want = qo.matmul_int4_int4t_int32(a, b, via='fp32')
+    got = quest.matmul_int4_int4t_int32(a.to(DEV), b.to(DEV)).cpu()
+    assert torch.equal(got, want)
+
+
+def test_matmul_int32_extreme_codes(quest):
+    # every product is (-8)(-8) = +64: the largest accumulator the path can see
+    m, k, n = 64, 4096, 96
+    a = torch.full((m, k // 2), 0x88, dtype=torch.uint8)
+    b = torch.full((n, k // 2), 0x88, dtype=torch.uint8)
+    got = quest.matmul_int4_int4t_int32(a.to(DEV), b.to(DEV)).cpu()
+    assert (got == 64 * k).all()
+    b[:] = 0x77                        # (-8)(7) = -56
+    got = quest.matmul_int4_int4t_int32(a.to(DEV), b.to(DEV)).cpu()
+    assert (got == -56 * k).all()
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 768, 224), (16, 4096, 4096), (1, 11008, 4096), (257, 256, 301)])
+def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
+    m, k, n = shape
+    g = torch.Generator().manual_seed(6)
+    a, b = rand_codes(m, k, 7), rand_codes(n, k, 8)
+    a_mul = (torch.rand(m, 1, generator=g) * 0.09 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype)
+    a_add = qo.unpack_int4(a).to(torch.int32).sum(-1, keepdim=True).to(torch.int32)
+    b_add = qo.unpack_int4(b).to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2
+    want = qo.fused_matmul_dequantize_int4_int4t(a, b, a_add, b_add, a_mul, b_mul, via='fp32')
+    got = quest.fused_matmul_dequantize_int4_int4t_bf16(
+        a.to(DEV), b.to(DEV), a_add.to(DEV), b_add.to(DEV), a_mul.to(DEV), b_mul.to(DEV)).cpu()
+    assert got.dtype == dtype
+    assert torch.equal(bits(got), bits(want))
+    # <= 1e-2 relative against the fp64 value of the dequantised product (the north star's bar)
+    ref = qo.linear_fp64(qo.unpack_int4(a), a_mul, qo.unpack_int4(b), b_mul)
+    assert ((got.double() - ref).norm() / ref.norm()) < 1e-2
+
+
+# --------------------------------------------------------------------------- H1 / H2
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('scale', [181. / 2048., 2. ** -3.5])
+def test_hadamard128(quest, dtype, scale):
+    x = rand_act(48, 1024, dtype, seed=9)
+    got = quest.hadamard128(x.to(DEV), scale=scale).cpu()
+    assert torch.equal(bits(got), bits(qo.hadamard128_fwht(x, scale)))      # same butterfly order
+    if scale == 181. / 2048.:
+        ref = qo.hadamard128_matmul(x)                                       # the reference's F.linear form
+        assert ((got.double() - ref.double()).norm() / ref.double().norm()) < 1e-3
+        # element-wise: the two summation orders differ by fp32 noise, i.e. at most one 16-bit ulp of
+        # the row's largest output (cancelled-out small outputs may be several of their own ulps apart)
+        tol = ref.double().abs().amax(-1, keepdim=True) * 2. ** -8
+        assert ((got.double() - ref.double()).abs() <= tol).all()
+    # in place
+    gx = x.to(DEV)
+    quest.hadamard128(gx, out=gx, scale=scale)
+    assert torch.equal(bits(gx.cpu()), bits(got))
+
+
+# --------------------------------------------------------------------------- fused activation kernel
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 768), (64, 4096), (1, 128), (8, 11008), (16, 2816), (2, 16384), (2, 32768)])
+def test_hadamard_quantize_fused(quest, dtype, shape):
+    m, k = shape
+    x = rand_act(m, k, dtype, seed=10)
+    gx = x.to(DEV)
+    x_had = torch.empty_like(gx)
+    scale, packed, row_sum = quest.hadamard_quantize_int4(gx, x_had=x_had)
+    assert torch.equal(bits(gx.cpu()), bits(x)), 'input must not be written'
+    # (1) Hadamard: bit-identical to the fp32-butterfly oracle, <= 1e-3 from the matmul formulation
+    want_had = qo.hadamard128_fwht(x, 181. / 2048.)
+    assert torch.equal(bits(x_had.cpu()), bits(want_had))
+    ref_had = qo.hadamard128_matmul(x)
+    assert ((want_had.double() - ref_had.double()).norm() / ref_had.double().norm()) < 1e-3
+    # (2) scale on that tensor: within one ulp of the oracle, rarely different
+    want_scale = qo.find_scale_int4(want_had)
+    d = ulp_diff(scale, want_scale)
+    assert d.max() <= 1 and (d != 0).sum() <= max(1, m // 100)
+    # (3) codes and row sums: bit-exact given the same transformed input and the same scale
+    xp = torch.empty(m, k // 2, dtype=torch.uint8)
+    rs = torch.empty(m, 1, dtype=torch.int32)
+    qo.quantize_int4(want_had, scale.cpu(), None, xp, rs, False)
+    assert torch.equal(packed.cpu(), xp)
+    assert torch.equal(row_sum.cpu(), rs)
+    # (4) the fusion equals its own unfused composition, bit for bit
+    h = quest.hadamard128(gx)
+    s2 = quest.find_scale_int4(h)
+    p2 = torch.empty_like(packed)
+    r2 = torch.empty_like(row_sum)
+    quest.quantize_int4(h, s2, None, p2, r2, False)
+    assert torch.equal(bits(s2.cpu()), bits(scale.cpu()))
+    assert torch.equal(p2, packed) and torch.equal(r2, row_sum)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_hadamard_quantize_without_hadamard(quest, dtype):
+    x = rand_act(40, 1024, dtype, seed=11)
+    scale, packed, row_sum = quest.hadamard_quantize_int4(x.to(DEV), hadamard_scale=0.)
+    want_scale = qo.find_scale_int4(x)
+    assert ulp_diff(scale, want_scale).max() <= 1
+    xp = torch.empty(40, 512, dtype=torch.uint8)
+    rs = torch.empty(40, 1, dtype=torch.int32)
+    qo.quantize_int4(x, scale.cpu(), None, xp, rs, False)
+    assert torch.equal(packed.cpu(), xp) and torch.equal(row_sum.cpu(), rs)
+
+
+def test_error_codes_no_launch(quest):
+    from quest_amd import _lib
+    lib = _lib.load()
+    x = torch.zeros(4, 128, dtype=torch.bfloat16, device=DEV)
+    s = torch.zeros(4, 1, dtype=torch.bfloat16, device=DEV)
+    st = _lib.stream_of(x)
+    assert lib.quest_find_scale_int4(None, _lib.ptr(x), 128, 4, 0, st) == -1
+    assert lib.quest_find_scale_int4(_lib.ptr(s), _lib.ptr(x), 100, 4, 0, st) == -2
+    assert lib.quest_find_scale_int4(_lib.ptr(s), _lib.ptr(x), 128, 4, 7, st) == -3
+    assert lib.quest_hadamard_quantize_int4(_lib.ptr(x), _lib.ptr(s), None, None, None, 64, 4, 0.1, 0, st) == -2
+    assert lib.quest_matmul_int4_int4t_int32(_lib.ptr(x), _lib.ptr(x), _lib.ptr(x), 4, 48, 4, st) == -2
+    with pytest.raises(RuntimeError):
+        quest.find_scale_int4(torch.zeros(2, 128, dtype=torch.bfloat16))       # CPU tensor: no fallback
+    with pytest.raises(NotImplementedError):
+        quest.matmul_int4sp_int4t_int32(None, None, None)
