@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A4 linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step is one W4A4 linear at the Llama-7B gate/up shape (M=4096 tokens, K=4096, N=11008): the
+fused Hadamard + scale + quantise + pack kernel on the fp16 activations, then the packed
+INT4 x INT4 GEMM with the scale epilogue to fp16.  Inputs are synthetic and already resident in
+HBM; several activation buffers are rotated so that no step finds its input in the Infinity Cache.
+`value` is 2*M*N*K / step time (TOPS of the whole linear, as the reference's published layer times
+are converted).  The JSON line also carries
+  roofline           the GEMM kernel against the INT8 MFMA peak (HIP-event time per launch),
+  roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
+                     outlier channels) against the HBM peak,
+  decode             the GEMM at M in {1, 8, 16}, weight streaming,
+  cpu_baseline       the CPU oracle (PyTorch restatement of the reference's `backend='pytorch'`
+                     path) on the reference's CPU-runnable case, timed on this host's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+INT8_MFMA_PEAK_TOPS = 5000.0
+
+# HBM bytes per launch read from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), scaled by a copy
+# kernel of known size; None until such a run has been recorded under profiles/.
+TRAFFIC_GEMM_BYTES = None
+TRAFFIC_QUANTIZE_BYTES = None
+
+
+def event_pairs(n):
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def mean_ms(pairs):
+    return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+
+
+def heavy_tailed_activations(m, k, dtype, device, seed):
+    """Student-t (3 degrees of freedom) entries, 1 % of the channels scaled by 20."""
+    g = torch.Generator(device='cpu').manual_seed(seed)
+    z = torch.randn(m, k, generator=g)
+    chi = torch.randn(m, k, 3, generator=g).square_().sum(-1)
+    x = z / (chi / 3).sqrt_()
+    cols = torch.randperm(k, generator=g)[: max(1, k // 100)]
+    x[:, cols] *= 20
+    return x.to(dtype).to(device)
+
+
+def bench_linear(quest, harness, steps, warmup, dev):
+    m, k, n = 4096, 4096, 11008
+    dtype = torch.float16
+    g = torch.Generator(device='cpu').manual_seed(0)
+    n_buf = 6
+    acts = [torch.randn(m, k, generator=g).to(dtype).to(dev) for _ in range(n_buf)]
+    # weights: uniform codes in [-8, 7], per-channel scales U(0.01, 0.1)
+    w_codes = torch.randint(-8, 8, (n, k), generator=g, dtype=torch.int8)
+    w_packed = ((w_codes[:, 1::2] << 4) | (w_codes[:, ::2] & 0xF)).view(torch.uint8).to(dev)
+    w_scale = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
+    w_add = (w_codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2).to(dev)
+    a_scale = torch.empty(m, 1, dtype=dtype, device=dev)
+    a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+    a_row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
+    out = torch.empty(m, n, dtype=dtype, device=dev)
+
+    def step(i, ev=None):
+        x = acts[i % n_buf]
+        if ev:
+            ev[0].record()
+        quest.hadamard_quantize_int4(x, a_scale, a_packed, a_row_sum)
+        if ev:
+            ev[1].record()
+        quest.fused_matmul_dequantize_int4_int4t_bf16(a_packed, w_packed, a_row_sum, w_add, a_scale, w_scale, out)
+        if ev:
+            ev[2].record()
+
+    for i in range(warmup):
+        step(i)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, evs[i])
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    quant_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    gemm_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    ops = 2.0 * m * n * k
+    return {
+        'shape': {'M': m, 'K': k, 'N': n},
+        'ms_per_step': ms_per_step,
+        'tops': ops / (ms_per_step * 1e-3) / 1e12,
+        'gemm_ms': gemm_ms,
+        'gemm_tops': ops / (gemm_ms * 1e-3) / 1e12,
+        'quant_ms': quant_ms,
+    }
+
+
+def bench_quantize(quest, steps, warmup, dev):
+    m, k = 8192, 4096
+    dtype = torch.bfloat16
+    n_buf = 6                                   # 6 x 64 MiB > the 256 MB Infinity Cache
+    xs = [heavy_tailed_activations(m, k, dtype, dev, seed=s) for s in range(n_buf)]
+    scale = torch.empty(m, 1, dtype=dtype, device=dev)
+    packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+    row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
+    for i in range(warmup):
+        quest.hadamard_quantize_int4(xs[i % n_buf], scale, packed, row_sum)
+    pairs = event_pairs(steps)
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(pairs):
+        a.record()
+        quest.hadamard_quantize_int4(xs[i % n_buf], scale, packed, row_sum)
+        b.record()
+    torch.cuda.synchronize()
+    ms = mean_ms(pairs)
+    algo_bytes = m * k * 2 + m * k // 2 + m * 2 + m * 4
+    gbs = algo_bytes / (ms * 1e-3) / 1e9
+    return {'bound': 'hbm', 'achieved': gbs, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs / HBM_PEAK_GBS,
+            'traffic': TRAFFIC_QUANTIZE_BYTES, 'kernel': 'hadamard_quantize_kernel', 'us_per_launch': ms * 1e3,
+            'algorithmic_bytes': algo_bytes, 'workload': 'bf16 [8192,4096] Student-t(3), 1% channels x20'}
+
+
+def bench_decode(quest, dev):
+    out = []
+    dtype = torch.float16
+    g = torch.Generator(device='cpu').manual_seed(1)
+    for k, n in [(4096, 4096), (11008, 4096)]:
+        n_w = 8                                  # rotate weight copies so they stream from HBM
+        ws = [torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.uint8).to(dev) for _ in range(n_w)]
+        w_scale = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
+        w_add = torch.randint(-500, 500, (n, 1), generator=g, dtype=torch.int32).to(dev)
+        for m in (1, 8, 16):
+            x = torch.randn(m, k, generator=g).to(dtype).to(dev)
+            a_scale = torch.empty(m, 1, dtype=dtype, device=dev)
+            a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+            a_row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
+            y = torch.empty(m, n, dtype=dtype, device=dev)
+
+            def run(i):
+                quest.hadamard_quantize_int4(x, a_scale, a_packed, a_row_sum)
+                quest.fused_matmul_dequantize_int4_int4t_bf16(a_packed, ws[i % n_w], a_row_sum, w_add, a_scale, w_scale, y)
+
+            for i in range(5):
+                run(i)
+            pairs = event_pairs(40)
+            torch.cuda.synchronize()
+            for i, (a, b) in enumerate(pairs):
+                a.record()
+                run(i)
+                b.record()
+            torch.cuda.synchronize()
+            us = mean_ms(pairs) * 1e3
+            wbytes = n * k // 2
+            out.append({'M': m, 'K': k, 'N': n, 'us': round(us, 2), 'weight_GBs': round(wbytes / us / 1e3, 1),
+                        'frac_hbm': round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+    return out
+
+
+def bench_cpu_baseline():
+    """The CPU oracle on the reference's CPU-runnable case: fp16 [512,1024] x [1024,1024]^T, Hadamard
+    as F.linear, scale, quantise, integer GEMM through fp64 as the reference's own check does, and
+    the scale epilogue."""
+    from oracle import quest_oracle as qo
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    m, k, n = 512, 1024, 1024
+    x = torch.randn(m, k).half()
+    w = (torch.randn(n, k) * 0.02).half()
+    wp, ws, wa, _ = qo.preprocess_weight(w, use_hadamard=True)
+    for _ in range(3):
+        qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='matmul', via='fp64')
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='matmul', via='fp64')
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    t32 = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='matmul', via='fp32')
+        t32.append(time.perf_counter() - t0)
+    t32.sort()
+    ops = 2.0 * m * n * k
+    return {'value': ops / med / 1e12, 'unit': 'TOPS', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'sample': f'W4A4 linear fp16 M={m} K={k} N={n}, seed 0, median of 10 calls after 3 warm-ups '
+                      f'({med * 1e3:.1f} ms per call; integer GEMM via fp64 matmul as the reference checks it)',
+            'ms_per_call': med * 1e3,
+            'faster_variant': {'what': 'same path with the integer GEMM as an exact fp32 matmul',
+                               'value': ops / t32[len(t32) // 2] / 1e12, 'ms_per_call': t32[len(t32) // 2] * 1e3}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py: this build runs on one GPU; --gpus above 1 is not supported '
+                 '(the path shards by tokens with no exchange, but no multi-GPU run is part of it)')
+    if not torch.cuda.is_available():
+        sys.exit('bench.py: no GPU visible')
+    import quest_amd as quest
+    from quest_amd import _lib, harness
+    _lib.load()
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+
+    lin = bench_linear(quest, harness, args.steps, args.warmup, dev)
+    rq = bench_quantize(quest, max(args.steps, 20), args.warmup, dev)
+    dec = bench_decode(quest, dev)
+    cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
+
+    roofline = {'bound': 'mfma', 'achieved': lin['gemm_tops'], 'peak': INT8_MFMA_PEAK_TOPS, 'unit': 'TOP/s',
+                'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES,
+                'kernel': 'gemm_w4a4_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
+                'algorithmic_ops': 2.0 * 4096 * 4096 * 11008}
+    line = {
+        'metric': 'INT4-GEMM TOPS + quantize GB/s at Llama-7B layer shapes, % MI355X roofline',
+        'value': lin['tops'], 'unit': 'TOPS', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': lin['ms_per_step'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'int8', 'data': 'synthetic',
+        'config': {'workload': 'W4A4 linear, Llama-7B gate/up: fp16 activations [4096,4096] -> fused '
+                               'Hadamard-quantize-pack -> packed INT4 GEMM [4096,4096]x[11008,4096]^T -> fp16 [4096,11008]',
+                   'M': 4096, 'K': 4096, 'N': 11008},
+        'gemm_tops': lin['gemm_tops'], 'quantize_us_in_step': lin['quant_ms'] * 1e3,
+        'quantize_GBs': rq['achieved'],
+        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'cpu_baseline': cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()
