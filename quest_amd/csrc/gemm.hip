@@ -485,6 +485,393 @@ gemm_w4a4_stream_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
 
 }  // namespace stream
 
+
+// =================================================================================================
+// Large-tile persistent kernel (K % 256 == 0): the prefill path
+// =================================================================================================
+// One workgroup of four waves per CU owns 256 tokens x up to 256 channels; wave w multiplies tokens
+// [128 (w >> 1), +128) by the lower or upper half of the tile's channel units (up to 128 x 128 per
+// wave: 4 x 4 accumulators in the AGPR half of the 512-register budget a single wave per SIMD has).
+// That halves the L2 -> CU traffic per multiply of the 128-channel kernel above.  Packed bytes go
+// HBM -> registers (two register sets, loads issued two stages ahead), are split into the two int8
+// vectors of 16 * nibble there -- once per byte instead of once per wave that uses it -- and
+// written to a double-buffered, XOR-swizzled int8 LDS tile.  The pipeline runs on across the
+// workgroup's tiles: the first stages of the next tile are loaded and staged while the last ones of
+// the current tile are multiplied, and the epilogue's stores drain under the next tile's first stages.
+namespace big {
+
+constexpr int kRows = 256;                    // rows of either operand per tile
+constexpr int kMaxUnits = 8;                  // channel units (32 rows) per tile
+constexpr int kRowB = 128;                    // int8 bytes per row per stage (128 k)
+constexpr int kTileB = kRows * kRowB;         // 32 KiB
+constexpr int kStageB = 2 * kTileB;           // token tile + channel tile
+constexpr int kVecB = 2 * (kRows * 4 + kRows * 2);   // two parities of (b_add int32, b_mul 16-bit) per channel
+constexpr int kLdsB = 2 * kStageB + kVecB;    // 131 KiB of the CU's 160 KiB
+
+// position of 16-byte chunk u of row r inside its 128-byte LDS row is u ^ chunk_swz(r): conflict-free
+// for the staging writes (8 lanes: 2 rows x 4 packed chunks) and for the operand reads (rows li, li + 1 ...)
+__device__ __forceinline__ int chunk_swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+
+struct Cursor {          // walks a workgroup's run of cells tile by tile, stage by stage (no divisions)
+    int tt, u;               // next cell: token tile, channel unit inside the group
+    int left;                // cells left in the run
+    int nug, ug0;
+    int tok0, ch0, width;    // current tile
+    int kt;                  // next stage of the current tile
+    bool valid;
+};
+
+__device__ __forceinline__ void cursor_next_tile(Cursor &c) {
+    if (c.left <= 0) { c.valid = false; return; }             // keeps pointing at the last tile
+    int width = c.nug - c.u;
+    width = width < c.left ? width : c.left;
+    width = width < kMaxUnits ? width : kMaxUnits;
+    c.tok0 = c.tt * kRows;
+    c.ch0 = (c.ug0 + c.u) * 32;
+    c.width = width;
+    c.kt = 0;
+    c.valid = true;
+    c.left -= width;
+    c.u += width;
+    if (c.u == c.nug) { c.u = 0; c.tt++; }
+}
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+struct Stager {           // per-thread staging state: thread t handles packed chunk t & 3 of rows (t >> 2) + 64 i
+    v4u ga[8], gb[8];     // i = 0..3 token rows, 4..7 channel rows
+    uint32_t off_t, off_c;   // byte offsets of row (t >> 2) of the load cursor's tile from the matrix bases
+    int st_e, st_o, srow, sq;
+};
+
+__device__ __forceinline__ void stager_offsets(Stager &s, const Cursor &ld, int kbytes) {
+    s.off_t = (uint32_t)(ld.tok0 + s.srow) * (uint32_t)kbytes + s.sq * 16;
+    s.off_c = (uint32_t)(ld.ch0 + s.srow) * (uint32_t)kbytes + s.sq * 16;
+}
+
+// Fetch the load cursor's stage into g, then advance the cursor (into the next tile when this one is
+// done).  Rows past the end of a matrix are out of the buffer's range and read as zeros.
+__device__ __forceinline__ void stager_gload(Stager &s, v4u (&g)[8], Cursor &ld, __amdgpu_buffer_rsrc_t act,
+                                             __amdgpu_buffer_rsrc_t wgt, int kbytes, int nk) {
+    const int kb = ld.kt * 64;
+    const int step = 64 * kbytes;
+#pragma unroll
+    for (int i = 0; i < 4; i++) g[i] = __builtin_amdgcn_raw_buffer_load_b128(act, s.off_t, kb + i * step, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) g[4 + i] = __builtin_amdgcn_raw_buffer_load_b128(wgt, s.off_c, kb + i * step, 0);
+    if (++ld.kt == nk) {
+        cursor_next_tile(ld);
+        if (ld.valid) stager_offsets(s, ld, kbytes); else ld.kt = nk - 1;   // nothing left: re-read the last stage
+    }
+}
+
+__device__ __forceinline__ void stager_store(const Stager &s, const v4u (&g)[8], uint8_t *lds, int buf, int first, int count) {
+    uint8_t *sb = lds + buf * kStageB + s.srow * kRowB;
+#pragma unroll
+    for (int i = first; i < first + count; i++) {
+        const v4u v = g[i];
+        const v4u e = (v << 4) & 0xF0F0F0F0u;
+        const v4u o = v & 0xF0F0F0F0u;
+        uint8_t *base = sb + (i >> 2) * kTileB + (i & 3) * 64 * kRowB;
+        *reinterpret_cast<v4u *>(base + s.st_e) = e;
+        *reinterpret_cast<v4u *>(base + s.st_o) = o;
+    }
+}
+
+template <int OUT, int NA>
+__device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Stager &sg, void *__restrict__ out,
+                                         __amdgpu_buffer_rsrc_t act, __amdgpu_buffer_rsrc_t wgt,
+                                         const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
+                                         const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
+                                         int M, int N, int K, int tok0, int ch0, int unit0, int vec_par) {
+    constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wt = wave >> 1;
+    const int li = lane & 31;
+    const int lg = lane >> 5;
+    const int kbytes = K >> 1;
+    const int nk = K / 128;
+
+    // operand reads: row li of a 32-row sub-tile; k-step ks takes chunk 2 ks (lanes 0-31) or 2 ks + 1 (lanes 32-63)
+    const int rd0 = li * kRowB + ((lg ^ chunk_swz(li)) << 4);      // k-step ks: rd0 ^ (ks << 5)
+    const int t_base = (wt * 128) * kRowB;
+    const int c_base = kTileB + (unit0 * 32) * kRowB;
+
+    v16i acc[NA > 0 ? NA : 1][4];
+#pragma unroll
+    for (int a = 0; a < NA; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
+
+    // per-channel epilogue vectors of this tile -> LDS (read back after the K loop)
+    int32_t *v_add = reinterpret_cast<int32_t *>(lds + 2 * kStageB + vec_par * (kRows * 6));
+    uint16_t *v_mul = reinterpret_cast<uint16_t *>(lds + 2 * kStageB + vec_par * (kRows * 6) + kRows * 4);
+    if constexpr (OUT != OUT_INT32) {
+        int c = ch0 + tid;
+        c = c < N ? c : N - 1;
+        v_add[tid] = b_add[c];
+        v_mul[tid] = b_mul[c];
+    }
+
+    v4i tf[2][4], cf[2][NA > 0 ? NA : 1];
+    auto frag_load = [&](int fb, int buf, int ks) {
+        const uint8_t *sb = lds + buf * kStageB + (rd0 ^ (ks << 5));
+#pragma unroll
+        for (int b = 0; b < 4; b++) tf[fb][b] = *reinterpret_cast<const v4i *>(sb + t_base + b * 32 * kRowB);
+#pragma unroll
+        for (int a = 0; a < NA; a++) cf[fb][a] = *reinterpret_cast<const v4i *>(sb + c_base + a * 32 * kRowB);
+    };
+    auto mfma_step = [&](int fb) {
+#pragma unroll
+        for (int a = 0; a < NA; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cf[fb][a], tf[fb][b], acc[a][b], 0, 0, 0);
+    };
+
+    // Invariant at the top of an even stage kt: LDS buffer 0 holds stage kt, register set gb stage kt + 1
+    // (in flight), set ga stage kt + 2 (in flight).  Stages past this tile's last belong to the next tile.
+    frag_load(0, 0, 0);
+    for (int kt = 0; kt < nk; kt += 2) {
+        // ---- even stage: multiply buffer 0, stage gb -> buffer 1, refill gb
+        frag_load(1, 0, 1);
+        stager_store(sg, sg.gb, lds, 1, 0, 2);
+        mfma_step(0);
+        __builtin_amdgcn_sched_barrier(0);
+        frag_load(0, 0, 2);
+        stager_store(sg, sg.gb, lds, 1, 2, 3);
+        mfma_step(1);
+        __builtin_amdgcn_sched_barrier(0);
+        frag_load(1, 0, 3);
+        stager_store(sg, sg.gb, lds, 1, 5, 3);
+        mfma_step(0);
+        __builtin_amdgcn_sched_barrier(0);
+        stager_gload(sg, sg.gb, ld, act, wgt, kbytes, nk);
+        mfma_step(1);
+        lds_fence_barrier();
+        // ---- odd stage: multiply buffer 1, stage ga -> buffer 0, refill ga
+        frag_load(0, 1, 0);
+        frag_load(1, 1, 1);
+        stager_store(sg, sg.ga, lds, 0, 0, 2);
+        mfma_step(0);
+        __builtin_amdgcn_sched_barrier(0);
+        frag_load(0, 1, 2);
+        stager_store(sg, sg.ga, lds, 0, 2, 3);
+        mfma_step(1);
+        __builtin_amdgcn_sched_barrier(0);
+        frag_load(1, 1, 3);
+        stager_store(sg, sg.ga, lds, 0, 5, 3);
+        mfma_step(0);
+        __builtin_amdgcn_sched_barrier(0);
+        stager_gload(sg, sg.ga, ld, act, wgt, kbytes, nk);
+        mfma_step(1);
+        lds_fence_barrier();
+        frag_load(0, 0, 0);                 // first k-step of the next even stage (or of the next tile)
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------------------
+    // Accumulator register r of lane (li, lg) is channel 8 (r/4) + 4 lg + r%4 of token li: a lane owns
+    // 4 consecutive channels.  Storing those directly would write 16-byte pieces of each output row,
+    // which HBM can only take as read-modify-write.  Each wave therefore passes 32 tokens x its
+    // channels through LDS buffer 1 (free until the next tile's first stage is staged) and writes the
+    // rows back out as 16 bytes per lane, 16 lanes per 256-byte run.
+    constexpr int kEs = OUT == OUT_INT32 ? 4 : 2;                  // bytes per output element
+    constexpr int kEpiStride = 128 * kEs + (OUT == OUT_INT32 ? 16 : 8);
+    constexpr int kEpiWaveB = 32 * kEpiStride;
+    const bool fast = (N % (16 / kEs)) == 0;
+    if (NA > 0 && fast) {
+        uint8_t *ebuf = lds + kStageB + wave * kEpiWaveB;
+        constexpr int kChunksPerRow = (NA > 0 ? NA : 1) * 32 * kEs / 16;
+        constexpr int kChunks = 32 * kChunksPerRow;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int tok_w = tok0 + wt * 128 + b * 32 + li;      // the token whose values this lane converts
+            int t_add = 0;
+            float t_half_mul = 0.f;
+            if constexpr (OUT != OUT_INT32) {
+                const int tc = tok_w < M ? tok_w : M - 1;
+                t_add = a_add[tc];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(a_mul[tc]));
+            }
+#pragma unroll
+            for (int a = 0; a < NA; a++) {
+#pragma unroll
+                for (int rg = 0; rg < 4; rg++) {
+                    const int col = a * 32 + rg * 8 + lg * 4;         // channel inside this wave's half
+                    int c[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) c[e] = acc[a][b][rg * 4 + e] >> 8;
+                    uint8_t *dst = ebuf + li * kEpiStride + col * kEs;
+                    if constexpr (OUT == OUT_INT32) {
+                        *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+                    } else {
+                        const int cl = unit0 * 32 + col;
+                        const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
+                        const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
+                        const int adds[4] = {va.x, va.y, va.z, va.w};
+                        const float muls[4] = {lo_f32<DT>(vm.x), hi_f32<DT>(vm.x), lo_f32<DT>(vm.y), hi_f32<DT>(vm.y)};
+                        uint32_t h[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float lhs = (float)(c[e] * 2 + t_add + adds[e]);
+                            const float rhs = __fmul_rn(t_half_mul, muls[e]);
+                            h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
+                        }
+                        *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                    }
+                }
+            }
+            // rows back out: chunk idx -> (row, 16-byte piece of the row)
+#pragma unroll
+            for (int i = 0; i < (kChunks + 63) / 64; i++) {
+                const int idx = i * 64 + lane;
+                const int row = idx / kChunksPerRow;
+                const int ck = idx % kChunksPerRow;
+                const int tok = tok0 + wt * 128 + b * 32 + row;
+                const int ch = ch0 + unit0 * 32 + ck * (16 / kEs);
+                if (idx < kChunks && tok < M && ch < N) {
+                    const uint4 v = *reinterpret_cast<const uint4 *>(ebuf + row * kEpiStride + ck * 16);
+                    *reinterpret_cast<uint4 *>(reinterpret_cast<uint8_t *>(out) + ((size_t)tok * N + ch) * kEs) = v;
+                }
+            }
+        }
+    } else {
+        const bool vec_ok = (N & 3) == 0;
+    #pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int tok = tok0 + wt * 128 + b * 32 + li;
+            if (tok >= M) continue;
+            int t_add = 0;
+            float t_half_mul = 0.f;
+            if constexpr (OUT != OUT_INT32) {
+                t_add = a_add[tok];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(a_mul[tok]));
+            }
+    #pragma unroll
+            for (int a = 0; a < NA; a++) {
+    #pragma unroll
+                for (int rg = 0; rg < 4; rg++) {
+                    const int cl = (unit0 + a) * 32 + rg * 8 + lg * 4;        // channel inside the tile
+                    const int ch = ch0 + cl;
+                    if (ch >= N) continue;
+                    int c[4];
+    #pragma unroll
+                    for (int e = 0; e < 4; e++) c[e] = acc[a][b][rg * 4 + e] >> 8;
+                    const size_t o = (size_t)tok * N + ch;
+                    if constexpr (OUT == OUT_INT32) {
+                        int32_t *dst = reinterpret_cast<int32_t *>(out) + o;
+                        if (vec_ok) {
+                            *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+                        } else {
+    #pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (ch + e < N) dst[e] = c[e];
+                        }
+                    } else {
+                        const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
+                        const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
+                        const int adds[4] = {va.x, va.y, va.z, va.w};
+                        const float muls[4] = {lo_f32<DT>(vm.x), hi_f32<DT>(vm.x), lo_f32<DT>(vm.y), hi_f32<DT>(vm.y)};
+                        uint32_t h[4];
+    #pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float lhs = (float)(c[e] * 2 + t_add + adds[e]);
+                            const float rhs = __fmul_rn(t_half_mul, muls[e]);
+                            h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
+                        }
+                        uint16_t *dst = reinterpret_cast<uint16_t *>(out) + o;
+                        if (vec_ok) {
+                            *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                        } else {
+    #pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (ch + e < N) dst[e] = (uint16_t)h[e];
+                        }
+                    }
+                }
+            }
+        }
+    }
+    lds_fence_barrier();      // buffer 1 is staged again at the start of the next tile
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(256)
+gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
+                     const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
+                     const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
+                     int M, int N, int K, stream::Schedule sch) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsB];
+    const int tid = threadIdx.x;
+    // wave-uniform by construction; readfirstlane tells the compiler so, which keeps everything that is
+    // updated under `switch (na)` below (the load cursor, buffer offsets) in scalar registers
+    const int wc = __builtin_amdgcn_readfirstlane((tid >> 6) & 1);   // channel half this wave multiplies
+    const int kbytes = K >> 1;
+    const int nk = K / 128;
+    // raw buffer views of the two packed matrices: 32-bit offsets, no 64-bit address registers
+    const __amdgpu_buffer_rsrc_t act_rs = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, M * kbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wgt_rs = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, N * kbytes, 0x00020000);
+
+    const int grp = blockIdx.x % sch.groups;
+    const int rank = blockIdx.x / sch.groups;
+    const int per_grp = gridDim.x / sch.groups;
+    const int ug0 = (int)(((long)grp * sch.units) / sch.groups);
+    const int ug1 = (int)(((long)(grp + 1) * sch.units) / sch.groups);
+    Cursor cc, ld;
+    cc.nug = ug1 - ug0;
+    cc.ug0 = ug0;
+    const long cells = (long)sch.tiles_t * cc.nug;
+    const long pos0 = (cells * rank) / per_grp;
+    const long pos1 = (cells * (rank + 1)) / per_grp;
+    cc.tt = (int)(pos0 / cc.nug);
+    cc.u = (int)(pos0 % cc.nug);
+    cc.left = (int)(pos1 - pos0);
+    cc.valid = false;
+    cc.tok0 = cc.ch0 = cc.width = cc.kt = 0;
+    ld = cc;
+    cursor_next_tile(cc);
+    if (!cc.valid) return;                       // uniform: the whole workgroup has nothing to do
+    cursor_next_tile(ld);
+
+    // ---- pipeline prologue: stage 0 -> LDS buffer 0, stage 1 -> gb, stage 2 -> ga ----------------------
+    Stager sg;
+    sg.srow = tid >> 2;
+    sg.sq = tid & 3;
+    sg.st_e = ((2 * sg.sq) ^ chunk_swz(sg.srow)) * 16;
+    sg.st_o = ((2 * sg.sq + 1) ^ chunk_swz(sg.srow)) * 16;
+    stager_offsets(sg, ld, kbytes);
+    stager_gload(sg, sg.ga, ld, act_rs, wgt_rs, kbytes, nk);
+    stager_gload(sg, sg.gb, ld, act_rs, wgt_rs, kbytes, nk);
+    stager_store(sg, sg.ga, lds, 0, 0, 8);
+    stager_gload(sg, sg.ga, ld, act_rs, wgt_rs, kbytes, nk);
+    lds_fence_barrier();
+
+    int vec_par = 0;
+    while (cc.valid) {
+        const int h0 = (cc.width + 1) >> 1;
+        const int na = wc == 0 ? h0 : cc.width - h0;
+        const int unit0 = wc == 0 ? 0 : h0;
+#define QUEST_BIG_TILE(NA) \
+    big_tile<OUT, NA>(lds, ld, sg, out, act_rs, wgt_rs, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, vec_par)
+        switch (na) {
+            case 4: QUEST_BIG_TILE(4); break;
+            case 3: QUEST_BIG_TILE(3); break;
+            case 2: QUEST_BIG_TILE(2); break;
+            case 1: QUEST_BIG_TILE(1); break;
+            default: QUEST_BIG_TILE(0); break;
+        }
+#undef QUEST_BIG_TILE
+        vec_par ^= 1;
+        cursor_next_tile(cc);
+    }
+}
+
+}  // namespace big
+
 static int device_cu_count() {
     static int cus = 0;
     if (cus == 0) {
@@ -513,8 +900,24 @@ static int gemm_launch_stream(void *out, const uint8_t *a, const uint8_t *b, con
 }
 
 template <int OUT>
+static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
+                           const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    stream::Schedule sch;
+    sch.tiles_t = (M + big::kRows - 1) / big::kRows;
+    sch.units = (N + 31) / 32;
+    const long cells = (long)sch.tiles_t * sch.units;
+    long grid = device_cu_count();                          // one workgroup per CU
+    if (grid > cells) grid = cells;
+    sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
+    big::gemm_w4a4_big_kernel<OUT><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
+    return launch_status();
+}
+
+template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    if ((K & 255) == 0 && M > 64) return gemm_launch_big<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
