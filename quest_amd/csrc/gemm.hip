@@ -487,30 +487,41 @@ gemm_w4a4_stream_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
 
 
 // =================================================================================================
-// Large-tile persistent kernel (K % 256 == 0): the prefill path
+// Large-tile persistent kernel (K % 128 == 0): the prefill path
 // =================================================================================================
 // One workgroup of four waves per CU owns 256 tokens x up to 256 channels; wave w multiplies tokens
 // [128 (w >> 1), +128) by the lower or upper half of the tile's channel units (up to 128 x 128 per
-// wave: 4 x 4 accumulators in the AGPR half of the 512-register budget a single wave per SIMD has).
-// That halves the L2 -> CU traffic per multiply of the 128-channel kernel above.  Packed bytes go
-// HBM -> registers (two register sets, loads issued two stages ahead), are split into the two int8
-// vectors of 16 * nibble there -- once per byte instead of once per wave that uses it -- and
-// written to a double-buffered, XOR-swizzled int8 LDS tile.  The pipeline runs on across the
-// workgroup's tiles: the first stages of the next tile are loaded and staged while the last ones of
-// the current tile are multiplied, and the epilogue's stores drain under the next tile's first stages.
+// wave: 4 x 4 accumulators in the AGPR half of the 512 registers a lone wave per SIMD has).
+// Compared with the 128-channel kernel above this halves the L2 -> CU bytes per multiply, and
+// compared with staging int8 through registers it keeps the LDS pipe (the measured bottleneck of
+// that variant) at a third of the traffic: packed bytes go HBM -> LDS directly
+// (buffer_load_dwordx4 ... lds, four stages of 32 KiB), a lane reads 16 packed bytes of one row
+// and splits them into the int8 vectors of 16 * (even-k nibbles) and 16 * (odd-k nibbles), which
+// feed two MFMA k-steps.  The stage pipeline runs on across the workgroup's tiles, and the
+// epilogue's stores are left to drain under the next tile's first stages.
 namespace big {
 
 constexpr int kRows = 256;                    // rows of either operand per tile
 constexpr int kMaxUnits = 8;                  // channel units (32 rows) per tile
-constexpr int kRowB = 128;                    // int8 bytes per row per stage (128 k)
-constexpr int kTileB = kRows * kRowB;         // 32 KiB
+constexpr int kRowB = 64;                     // packed bytes per row per stage (128 k)
+constexpr int kTileB = kRows * kRowB;         // 16 KiB
 constexpr int kStageB = 2 * kTileB;           // token tile + channel tile
+constexpr int kStages = 4;
+constexpr int kLoads = 8;                     // buffer loads per wave per stage
+constexpr int kEpiStride = 136;               // bytes per token row of the epilogue transposition buffer
+constexpr int kEpiWaveB = 32 * kEpiStride;
+constexpr int kEpiOff = kStages * kStageB;
+constexpr int kVecOff = kEpiOff + 4 * kEpiWaveB;
 constexpr int kVecB = 2 * (kRows * 4 + kRows * 2);   // two parities of (b_add int32, b_mul 16-bit) per channel
-constexpr int kLdsB = 2 * kStageB + kVecB;    // 131 KiB of the CU's 160 KiB
+constexpr int kLdsB = kVecOff + kVecB;        // ~148 KiB of the CU's 160 KiB
 
-// position of 16-byte chunk u of row r inside its 128-byte LDS row is u ^ chunk_swz(r): conflict-free
-// for the staging writes (8 lanes: 2 rows x 4 packed chunks) and for the operand reads (rows li, li + 1 ...)
-__device__ __forceinline__ int chunk_swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+// s_barrier alone: waves order their own LDS traffic with s_waitcnt, and a release / acquire fence here would
+// make the compiler drain every direct-to-LDS load still in flight (vmcnt(0)), which is the pipeline
+__device__ __forceinline__ void plain_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 struct Cursor {          // walks a workgroup's run of cells tile by tile, stage by stage (no divisions)
     int tt, u;               // next cell: token tile, channel unit inside the group
@@ -536,70 +547,100 @@ __device__ __forceinline__ void cursor_next_tile(Cursor &c) {
     if (c.u == c.nug) { c.u = 0; c.tt++; }
 }
 
-typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-
-struct Stager {           // per-thread staging state: thread t handles packed chunk t & 3 of rows (t >> 2) + 64 i
-    v4u ga[8], gb[8];     // i = 0..3 token rows, 4..7 channel rows
-    uint32_t off_t, off_c;   // byte offsets of row (t >> 2) of the load cursor's tile from the matrix bases
-    int st_e, st_o, srow, sq;
+struct Loader {          // direct-to-LDS loads of one wave: 4 instructions of 16 token rows, 4 of 16 channel rows
+    __amdgpu_buffer_rsrc_t act, wgt, badd, bmul;
+    uint32_t off_t, off_c;      // byte offset of this lane's first row of the load cursor's tile (+ its 16-byte chunk)
+    int kbytes, nk, wave;
+    int issued;                 // stages issued so far by this workgroup (slot = issued % kStages)
 };
 
-__device__ __forceinline__ void stager_offsets(Stager &s, const Cursor &ld, int kbytes) {
-    s.off_t = (uint32_t)(ld.tok0 + s.srow) * (uint32_t)kbytes + s.sq * 16;
-    s.off_c = (uint32_t)(ld.ch0 + s.srow) * (uint32_t)kbytes + s.sq * 16;
+__device__ __forceinline__ void loader_offsets(Loader &l, const Cursor &ld, int lane) {
+    // lane p of an instruction covers row p / 4 of its 16 rows; LDS slot p (lane order) must hold chunk
+    // (p & 3) ^ ((row >> 2) & 3) of that row, so the lane fetches exactly that chunk
+    const int row = l.wave * 64 + (lane >> 2);
+    const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    l.off_t = (uint32_t)(ld.tok0 + row) * (uint32_t)l.kbytes + chunk * 16;
+    l.off_c = (uint32_t)(ld.ch0 + row) * (uint32_t)l.kbytes + chunk * 16;
 }
 
-// Fetch the load cursor's stage into g, then advance the cursor (into the next tile when this one is
-// done).  Rows past the end of a matrix are out of the buffer's range and read as zeros.
-__device__ __forceinline__ void stager_gload(Stager &s, v4u (&g)[8], Cursor &ld, __amdgpu_buffer_rsrc_t act,
-                                             __amdgpu_buffer_rsrc_t wgt, int kbytes, int nk) {
-    const int kb = ld.kt * 64;
-    const int step = 64 * kbytes;
+// Issue the load cursor's stage into the next LDS slot, then advance the cursor (into the next tile
+// when this one is done; when nothing is left the last stage is fetched again, which keeps the
+// count of outstanding loads uniform).  Rows past the end of a matrix read as zeros.
+__device__ __forceinline__ void loader_issue(Loader &l, Cursor &ld, uint8_t *lds, int lane) {
+    uint8_t *sb = lds + (l.issued % kStages) * kStageB + l.wave * 64 * kRowB;
+    const int kb = ld.kt * kRowB;
+    const int step = 16 * l.kbytes;
 #pragma unroll
-    for (int i = 0; i < 4; i++) g[i] = __builtin_amdgcn_raw_buffer_load_b128(act, s.off_t, kb + i * step, 0);
+    for (int j = 0; j < 4; j++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.act, (__attribute__((address_space(3))) void *)(sb + j * 16 * kRowB), 16,
+                                                 l.off_t, kb + j * step, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; i++) g[4 + i] = __builtin_amdgcn_raw_buffer_load_b128(wgt, s.off_c, kb + i * step, 0);
-    if (++ld.kt == nk) {
+    for (int j = 0; j < 4; j++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.wgt, (__attribute__((address_space(3))) void *)(sb + kTileB + j * 16 * kRowB),
+                                                 16, l.off_c, kb + j * step, 0, 0);
+    l.issued++;
+    if (++ld.kt == l.nk) {
         cursor_next_tile(ld);
-        if (ld.valid) stager_offsets(s, ld, kbytes); else ld.kt = nk - 1;   // nothing left: re-read the last stage
+        if (ld.valid) loader_offsets(l, ld, lane); else ld.kt = l.nk - 1;
     }
 }
 
-__device__ __forceinline__ void stager_store(const Stager &s, const v4u (&g)[8], uint8_t *lds, int buf, int first, int count) {
-    uint8_t *sb = lds + buf * kStageB + s.srow * kRowB;
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_imm() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));   // vmcnt only
+}
+// at most kLoads * (kStages - 3) + extra younger memory operations may still be in flight
+__device__ __forceinline__ void wait_stage(int extra) {
+    constexpr int kBase = kLoads * (kStages - 3);
+    switch (extra) {
+        case 34: wait_vmcnt_imm<kBase + 34>(); break;
+        case 26: wait_vmcnt_imm<kBase + 26>(); break;
+        case 18: wait_vmcnt_imm<kBase + 18>(); break;
+        case 10: wait_vmcnt_imm<kBase + 10>(); break;
+        case 2: wait_vmcnt_imm<kBase + 2>(); break;
+        default: wait_vmcnt_imm<kBase>(); break;
+    }
+}
+
+struct Pipe {            // state that lives across tiles
+    int it;              // stages multiplied so far (slot = it % kStages)
+    int store_extra;     // epilogue stores that may still be in flight ...
+    int store_syncs;     // ... for this many more stage synchronisations
+    int vec_par;
+};
+
+__device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
 #pragma unroll
-    for (int i = first; i < first + count; i++) {
-        const v4u v = g[i];
-        const v4u e = (v << 4) & 0xF0F0F0F0u;
-        const v4u o = v & 0xF0F0F0F0u;
-        uint8_t *base = sb + (i >> 2) * kTileB + (i & 3) * 64 * kRowB;
-        *reinterpret_cast<v4u *>(base + s.st_e) = e;
-        *reinterpret_cast<v4u *>(base + s.st_o) = o;
+    for (int d = 0; d < 4; d++) {
+        even[d] = (int)(((uint32_t)p[d] << 4) & 0xF0F0F0F0u);
+        odd[d] = (int)((uint32_t)p[d] & 0xF0F0F0F0u);
     }
 }
 
 template <int OUT, int NA>
-__device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Stager &sg, void *__restrict__ out,
-                                         __amdgpu_buffer_rsrc_t act, __amdgpu_buffer_rsrc_t wgt,
-                                         const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
-                                         const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
-                                         int M, int N, int K, int tok0, int ch0, int unit0, int vec_par) {
+__device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, v4i (&pf)[8], v4i (&pg)[8],
+                                         void *__restrict__ out, const int32_t *__restrict__ a_add,
+                                         const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
+                                         const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0,
+                                         int unit0, int width) {
     constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
+    constexpr int NAX = NA > 0 ? NA : 1;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wt = wave >> 1;
     const int li = lane & 31;
     const int lg = lane >> 5;
-    const int kbytes = K >> 1;
     const int nk = K / 128;
 
-    // operand reads: row li of a 32-row sub-tile; k-step ks takes chunk 2 ks (lanes 0-31) or 2 ks + 1 (lanes 32-63)
-    const int rd0 = li * kRowB + ((lg ^ chunk_swz(li)) << 4);      // k-step ks: rd0 ^ (ks << 5)
-    const int t_base = (wt * 128) * kRowB;
-    const int c_base = kTileB + (unit0 * 32) * kRowB;
+    // operand reads: row li of a 32-row sub-tile; the 16-byte chunk 2 j + lg of its 64-byte stage row (k-pair j)
+    const int rd_t = (wt * 128 + li) * kRowB;
+    const int rd_c = kTileB + (unit0 * 32 + li) * kRowB;
+    int rd_j[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) rd_j[j] = ((2 * j + lg) ^ ((li >> 2) & 3)) * 16;
 
-    v16i acc[NA > 0 ? NA : 1][4];
+    v16i acc[NAX][4];
 #pragma unroll
     for (int a = 0; a < NA; a++)
 #pragma unroll
@@ -607,86 +648,76 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Stager &sg, v
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
 
-    // per-channel epilogue vectors of this tile -> LDS (read back after the K loop)
-    int32_t *v_add = reinterpret_cast<int32_t *>(lds + 2 * kStageB + vec_par * (kRows * 6));
-    uint16_t *v_mul = reinterpret_cast<uint16_t *>(lds + 2 * kStageB + vec_par * (kRows * 6) + kRows * 4);
+    // per-channel epilogue vectors of this tile -> LDS, also by direct loads (two per wave: its 64 channels
+    // of b_add and of b_mul); they are read back after the K loop.  Counted in pp.store_extra below.
+    int32_t *v_add = reinterpret_cast<int32_t *>(lds + kVecOff + pp.vec_par * (kRows * 6));
+    uint16_t *v_mul = reinterpret_cast<uint16_t *>(lds + kVecOff + pp.vec_par * (kRows * 6) + kRows * 4);
     if constexpr (OUT != OUT_INT32) {
-        int c = ch0 + tid;
-        c = c < N ? c : N - 1;
-        v_add[tid] = b_add[c];
-        v_mul[tid] = b_mul[c];
+        const int c = ch0 + wave * 64 + lane;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ldr.badd, (__attribute__((address_space(3))) void *)(v_add + wave * 64), 4,
+                                                 c * 4, 0, 0, 0);
+        // a direct load places lane l's data at 4 l bytes whatever its size, so b_mul travels as 32 dwords of two
+        if (lane < 32)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ldr.bmul, (__attribute__((address_space(3))) void *)(v_mul + wave * 64), 4,
+                                                     (ch0 + wave * 64 + 2 * lane) * 2, 0, 0, 0);
     }
 
-    v4i tf[2][4], cf[2][NA > 0 ? NA : 1];
-    auto frag_load = [&](int fb, int buf, int ks) {
-        const uint8_t *sb = lds + buf * kStageB + (rd0 ^ (ks << 5));
+    // packed operand fragments of one k-pair: pf[0..3] the four token sub-tiles, pf[4..] the channel sub-tiles
+    auto frag_read = [&](v4i (&f)[8], int slot, int j) {
+        const uint8_t *sb = lds + slot * kStageB + rd_j[j];
 #pragma unroll
-        for (int b = 0; b < 4; b++) tf[fb][b] = *reinterpret_cast<const v4i *>(sb + t_base + b * 32 * kRowB);
+        for (int b = 0; b < 4; b++) f[b] = *reinterpret_cast<const v4i *>(sb + rd_t + b * 32 * kRowB);
 #pragma unroll
-        for (int a = 0; a < NA; a++) cf[fb][a] = *reinterpret_cast<const v4i *>(sb + c_base + a * 32 * kRowB);
+        for (int a = 0; a < NA; a++) f[4 + a] = *reinterpret_cast<const v4i *>(sb + rd_c + a * 32 * kRowB);
     };
-    auto mfma_step = [&](int fb) {
+    // split the fragments in registers and run the two k-steps they hold
+    auto multiply = [&](const v4i (&f)[8]) {
+        v4i te[4], to[4];
 #pragma unroll
-        for (int a = 0; a < NA; a++)
+        for (int b = 0; b < 4; b++) split16(f[b], te[b], to[b]);
 #pragma unroll
-            for (int b = 0; b < 4; b++)
-                acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cf[fb][a], tf[fb][b], acc[a][b], 0, 0, 0);
+        for (int a = 0; a < NA; a++) {
+            v4i ce, co;
+            split16(f[4 + a], ce, co);
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te[b], acc[a][b], 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to[b], acc[a][b], 0, 0, 0);
+        }
     };
 
-    // Invariant at the top of an even stage kt: LDS buffer 0 holds stage kt, register set gb stage kt + 1
-    // (in flight), set ga stage kt + 2 (in flight).  Stages past this tile's last belong to the next tile.
-    frag_load(0, 0, 0);
-    for (int kt = 0; kt < nk; kt += 2) {
-        // ---- even stage: multiply buffer 0, stage gb -> buffer 1, refill gb
-        frag_load(1, 0, 1);
-        stager_store(sg, sg.gb, lds, 1, 0, 2);
-        mfma_step(0);
-        __builtin_amdgcn_sched_barrier(0);
-        frag_load(0, 0, 2);
-        stager_store(sg, sg.gb, lds, 1, 2, 3);
-        mfma_step(1);
-        __builtin_amdgcn_sched_barrier(0);
-        frag_load(1, 0, 3);
-        stager_store(sg, sg.gb, lds, 1, 5, 3);
-        mfma_step(0);
-        __builtin_amdgcn_sched_barrier(0);
-        stager_gload(sg, sg.gb, ld, act, wgt, kbytes, nk);
-        mfma_step(1);
-        lds_fence_barrier();
-        // ---- odd stage: multiply buffer 1, stage ga -> buffer 0, refill ga
-        frag_load(0, 1, 0);
-        frag_load(1, 1, 1);
-        stager_store(sg, sg.ga, lds, 0, 0, 2);
-        mfma_step(0);
-        __builtin_amdgcn_sched_barrier(0);
-        frag_load(0, 1, 2);
-        stager_store(sg, sg.ga, lds, 0, 2, 3);
-        mfma_step(1);
-        __builtin_amdgcn_sched_barrier(0);
-        frag_load(1, 1, 3);
-        stager_store(sg, sg.ga, lds, 0, 5, 3);
-        mfma_step(0);
-        __builtin_amdgcn_sched_barrier(0);
-        stager_gload(sg, sg.ga, ld, act, wgt, kbytes, nk);
-        mfma_step(1);
-        lds_fence_barrier();
-        frag_load(0, 0, 0);                 // first k-step of the next even stage (or of the next tile)
+    // On entry pf[0..3] hold the token fragments of (stage pp.it, k-pair 0), read by the previous tile's last
+    // stage (token rows do not depend on the tile); the channel rows do, so their fragments are read here.
+    {
+        const uint8_t *sb = lds + (pp.it % kStages) * kStageB + rd_j[0];
+#pragma unroll
+        for (int a = 0; a < NA; a++) pf[4 + a] = *reinterpret_cast<const v4i *>(sb + rd_c + a * 32 * kRowB);
+    }
+    for (int kt = 0; kt < nk; kt++) {
+        const int slot = pp.it % kStages;
+        frag_read(pg, slot, 1);                     // k-pair 1 of this stage
+        multiply(pf);
+        // stage pp.it + 1 must have landed everywhere before its first fragments are read below; the slot of
+        // stage pp.it - 1 is free for the loads of stage pp.it + kStages - 1 once everyone is past this barrier
+        if (pp.store_syncs > 0) { wait_stage(pp.store_extra); pp.store_syncs--; } else { wait_stage(0); }
+        plain_barrier();
+        loader_issue(ldr, ld, lds, lane);
+        frag_read(pf, (pp.it + 1) % kStages, 0);    // k-pair 0 of the next stage (maybe the next tile's)
+        multiply(pg);
+        pp.it++;
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
     // Accumulator register r of lane (li, lg) is channel 8 (r/4) + 4 lg + r%4 of token li: a lane owns
-    // 4 consecutive channels.  Storing those directly would write 16-byte pieces of each output row,
-    // which HBM can only take as read-modify-write.  Each wave therefore passes 32 tokens x its
-    // channels through LDS buffer 1 (free until the next tile's first stage is staged) and writes the
-    // rows back out as 16 bytes per lane, 16 lanes per 256-byte run.
+    // 4 consecutive channels.  Storing those directly would write 8- or 16-byte pieces of each output
+    // row.  Each wave instead passes 32 tokens x 64 channels (32 for int32) at a time through its own LDS
+    // strip and writes 128-byte runs of each row, 16 bytes per lane.
     constexpr int kEs = OUT == OUT_INT32 ? 4 : 2;                  // bytes per output element
-    constexpr int kEpiStride = 128 * kEs + (OUT == OUT_INT32 ? 16 : 8);
-    constexpr int kEpiWaveB = 32 * kEpiStride;
+    constexpr int kApp = OUT == OUT_INT32 ? 1 : 2;                 // channel sub-tiles per pass
     const bool fast = (N % (16 / kEs)) == 0;
+    const bool interior = fast && tok0 + kRows <= M && ch0 + 32 * width <= N;
     if (NA > 0 && fast) {
-        uint8_t *ebuf = lds + kStageB + wave * kEpiWaveB;
-        constexpr int kChunksPerRow = (NA > 0 ? NA : 1) * 32 * kEs / 16;
-        constexpr int kChunks = 32 * kChunksPerRow;
+        uint8_t *ebuf = lds + kEpiOff + wave * kEpiWaveB;
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             const int tok_w = tok0 + wt * 128 + b * 32 + li;      // the token whose values this lane converts
@@ -698,50 +729,59 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Stager &sg, v
                 t_half_mul = __fmul_rn(0.5f, to_f32<DT>(a_mul[tc]));
             }
 #pragma unroll
-            for (int a = 0; a < NA; a++) {
+            for (int a0 = 0; a0 < NA; a0 += kApp) {
+                constexpr int dummy = 0;
+                (void)dummy;
+                const int cnt = (NA - a0) < kApp ? (NA - a0) : kApp;
 #pragma unroll
-                for (int rg = 0; rg < 4; rg++) {
-                    const int col = a * 32 + rg * 8 + lg * 4;         // channel inside this wave's half
-                    int c[4];
+                for (int aa = 0; aa < kApp; aa++) {
+                    const int a = a0 + aa;
+                    if (a >= NA) continue;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) c[e] = acc[a][b][rg * 4 + e] >> 8;
-                    uint8_t *dst = ebuf + li * kEpiStride + col * kEs;
-                    if constexpr (OUT == OUT_INT32) {
-                        *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
-                    } else {
-                        const int cl = unit0 * 32 + col;
-                        const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
-                        const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
-                        const int adds[4] = {va.x, va.y, va.z, va.w};
-                        const float muls[4] = {lo_f32<DT>(vm.x), hi_f32<DT>(vm.x), lo_f32<DT>(vm.y), hi_f32<DT>(vm.y)};
-                        uint32_t h[4];
+                    for (int rg = 0; rg < 4; rg++) {
+                        const int col = aa * 32 + rg * 8 + lg * 4;            // channel inside this pass
+                        int c[4];
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const float lhs = (float)(c[e] * 2 + t_add + adds[e]);
-                            const float rhs = __fmul_rn(t_half_mul, muls[e]);
-                            h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
+                        for (int e = 0; e < 4; e++) c[e] = acc[a < NAX ? a : 0][b][rg * 4 + e] >> 8;
+                        uint8_t *dst = ebuf + li * kEpiStride + col * kEs;
+                        if constexpr (OUT == OUT_INT32) {
+                            *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+                        } else {
+                            const int cl = (unit0 + a) * 32 + rg * 8 + lg * 4;   // channel inside the tile
+                            const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
+                            const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
+                            const int adds[4] = {va.x, va.y, va.z, va.w};
+                            const float muls[4] = {lo_f32<DT>(vm.x), hi_f32<DT>(vm.x), lo_f32<DT>(vm.y), hi_f32<DT>(vm.y)};
+                            uint32_t h[4];
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const float lhs = (float)(c[e] * 2 + t_add + adds[e]);
+                                const float rhs = __fmul_rn(t_half_mul, muls[e]);
+                                h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
+                            }
+                            *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
                         }
-                        *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                    }
+                }
+                // rows back out: 32 rows x (cnt * 32 channels) in 16-byte pieces
+                const int pieces = cnt * 2 * kEs;
+#pragma unroll
+                for (int i = 0; i < kApp * kEs; i++) {
+                    const int idx = i * 64 + lane;
+                    const int row = idx / pieces;
+                    const int ck = idx - row * pieces;
+                    const int tok = tok0 + wt * 128 + b * 32 + row;
+                    const int ch = ch0 + (unit0 + a0) * 32 + ck * (16 / kEs);
+                    if (row < 32 && tok < M && ch < N) {
+                        const uint4 v = *reinterpret_cast<const uint4 *>(ebuf + row * kEpiStride + ck * 16);
+                        *reinterpret_cast<uint4 *>(reinterpret_cast<uint8_t *>(out) + ((size_t)tok * N + ch) * kEs) = v;
                     }
                 }
             }
-            // rows back out: chunk idx -> (row, 16-byte piece of the row)
-#pragma unroll
-            for (int i = 0; i < (kChunks + 63) / 64; i++) {
-                const int idx = i * 64 + lane;
-                const int row = idx / kChunksPerRow;
-                const int ck = idx % kChunksPerRow;
-                const int tok = tok0 + wt * 128 + b * 32 + row;
-                const int ch = ch0 + unit0 * 32 + ck * (16 / kEs);
-                if (idx < kChunks && tok < M && ch < N) {
-                    const uint4 v = *reinterpret_cast<const uint4 *>(ebuf + row * kEpiStride + ck * 16);
-                    *reinterpret_cast<uint4 *>(reinterpret_cast<uint8_t *>(out) + ((size_t)tok * N + ch) * kEs) = v;
-                }
-            }
         }
-    } else {
-        const bool vec_ok = (N & 3) == 0;
-    #pragma unroll
+    } else if (NA > 0) {
+        // generic path (N not a multiple of 8 / 4): element-wise stores straight from the accumulators
+#pragma unroll
         for (int b = 0; b < 4; b++) {
             const int tok = tok0 + wt * 128 + b * 32 + li;
             if (tok >= M) continue;
@@ -751,52 +791,40 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Stager &sg, v
                 t_add = a_add[tok];
                 t_half_mul = __fmul_rn(0.5f, to_f32<DT>(a_mul[tok]));
             }
-    #pragma unroll
+#pragma unroll
             for (int a = 0; a < NA; a++) {
-    #pragma unroll
+#pragma unroll
                 for (int rg = 0; rg < 4; rg++) {
-                    const int cl = (unit0 + a) * 32 + rg * 8 + lg * 4;        // channel inside the tile
-                    const int ch = ch0 + cl;
-                    if (ch >= N) continue;
-                    int c[4];
-    #pragma unroll
-                    for (int e = 0; e < 4; e++) c[e] = acc[a][b][rg * 4 + e] >> 8;
-                    const size_t o = (size_t)tok * N + ch;
-                    if constexpr (OUT == OUT_INT32) {
-                        int32_t *dst = reinterpret_cast<int32_t *>(out) + o;
-                        if (vec_ok) {
-                            *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+                    const int cl = (unit0 + a) * 32 + rg * 8 + lg * 4;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int ch = ch0 + cl + e;
+                        if (ch >= N) continue;
+                        const int c = acc[a][b][rg * 4 + e] >> 8;
+                        const size_t o = (size_t)tok * N + ch;
+                        if constexpr (OUT == OUT_INT32) {
+                            reinterpret_cast<int32_t *>(out)[o] = c;
                         } else {
-    #pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (ch + e < N) dst[e] = c[e];
-                        }
-                    } else {
-                        const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
-                        const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
-                        const int adds[4] = {va.x, va.y, va.z, va.w};
-                        const float muls[4] = {lo_f32<DT>(vm.x), hi_f32<DT>(vm.x), lo_f32<DT>(vm.y), hi_f32<DT>(vm.y)};
-                        uint32_t h[4];
-    #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const float lhs = (float)(c[e] * 2 + t_add + adds[e]);
-                            const float rhs = __fmul_rn(t_half_mul, muls[e]);
-                            h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
-                        }
-                        uint16_t *dst = reinterpret_cast<uint16_t *>(out) + o;
-                        if (vec_ok) {
-                            *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-                        } else {
-    #pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (ch + e < N) dst[e] = (uint16_t)h[e];
+                            const float lhs = (float)(c * 2 + t_add + v_add[cl + e]);
+                            const float rhs = __fmul_rn(t_half_mul, to_f32<DT>(v_mul[cl + e]));
+                            reinterpret_cast<uint16_t *>(out)[o] = (uint16_t)from_f32<DT>(__fmul_rn(lhs, rhs));
                         }
                     }
                 }
             }
         }
     }
-    lds_fence_barrier();      // buffer 1 is staged again at the start of the next tile
+    // how many of this wave's stores the next stage synchronisations may leave in flight: exact only when every
+    // store instruction of the fast path was issued with all its lanes (an interior tile), otherwise none
+    // (the next tile's two vector loads, issued right after this point, are always exact)
+    if constexpr (OUT != OUT_INT32) {
+        pp.store_extra = (interior ? 8 * NA : 0) + 2;
+        pp.store_syncs = kStages - 2;
+    } else {
+        pp.store_extra = 0;
+        pp.store_syncs = 0;
+    }
+    pp.vec_par ^= 1;
 }
 
 template <int OUT>
@@ -807,14 +835,12 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
                      int M, int N, int K, stream::Schedule sch) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsB];
     const int tid = threadIdx.x;
+    const int lane = tid & 63;
     // wave-uniform by construction; readfirstlane tells the compiler so, which keeps everything that is
-    // updated under `switch (na)` below (the load cursor, buffer offsets) in scalar registers
-    const int wc = __builtin_amdgcn_readfirstlane((tid >> 6) & 1);   // channel half this wave multiplies
+    // updated under `switch (na)` below (cursors, slot numbers, LDS bases) in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wc = wave & 1;                     // channel half this wave multiplies
     const int kbytes = K >> 1;
-    const int nk = K / 128;
-    // raw buffer views of the two packed matrices: 32-bit offsets, no 64-bit address registers
-    const __amdgpu_buffer_rsrc_t act_rs = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, M * kbytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t wgt_rs = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, N * kbytes, 0x00020000);
 
     const int grp = blockIdx.x % sch.groups;
     const int rank = blockIdx.x / sch.groups;
@@ -837,26 +863,45 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     if (!cc.valid) return;                       // uniform: the whole workgroup has nothing to do
     cursor_next_tile(ld);
 
-    // ---- pipeline prologue: stage 0 -> LDS buffer 0, stage 1 -> gb, stage 2 -> ga ----------------------
-    Stager sg;
-    sg.srow = tid >> 2;
-    sg.sq = tid & 3;
-    sg.st_e = ((2 * sg.sq) ^ chunk_swz(sg.srow)) * 16;
-    sg.st_o = ((2 * sg.sq + 1) ^ chunk_swz(sg.srow)) * 16;
-    stager_offsets(sg, ld, kbytes);
-    stager_gload(sg, sg.ga, ld, act_rs, wgt_rs, kbytes, nk);
-    stager_gload(sg, sg.gb, ld, act_rs, wgt_rs, kbytes, nk);
-    stager_store(sg, sg.ga, lds, 0, 0, 8);
-    stager_gload(sg, sg.ga, ld, act_rs, wgt_rs, kbytes, nk);
-    lds_fence_barrier();
+    Loader ldr;
+    ldr.act = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, M * kbytes, 0x00020000);
+    ldr.wgt = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, N * kbytes, 0x00020000);
+    ldr.badd = __builtin_amdgcn_make_buffer_rsrc((void *)b_add, 0, N * 4, 0x00020000);
+    ldr.bmul = __builtin_amdgcn_make_buffer_rsrc((void *)b_mul, 0, N * 2, 0x00020000);
+    ldr.kbytes = kbytes;
+    ldr.nk = K / 128;
+    ldr.wave = wave;
+    ldr.issued = 0;
+    loader_offsets(ldr, ld, lane);
 
-    int vec_par = 0;
+    // ---- pipeline prologue: stages 0 .. kStages - 2 in flight, fragments of (stage 0, k-pair 0) in registers
+#pragma unroll
+    for (int s = 0; s < kStages - 1; s++) loader_issue(ldr, ld, lds, lane);
+    wait_vmcnt_imm<kLoads * (kStages - 2)>();
+    plain_barrier();
+    Pipe pp;
+    pp.it = 0;
+    pp.store_extra = OUT != OUT_INT32 ? 2 : 0;   // the first tile's two vector loads
+    pp.store_syncs = OUT != OUT_INT32 ? kStages - 2 : 0;
+    pp.vec_par = 0;
+    v4i pf[8], pg[8];
+    {
+        const int li = lane & 31, lg = lane >> 5;
+        const uint8_t *sb = lds + ((0 + lg) ^ ((li >> 2) & 3)) * 16;
+#pragma unroll
+        for (int b = 0; b < 4; b++) pf[b] = *reinterpret_cast<const v4i *>(sb + ((wave >> 1) * 128 + li + b * 32) * kRowB);
+#pragma unroll
+        for (int a = 0; a < 4; a++) pf[4 + a] = pf[0];
+#pragma unroll
+        for (int i = 0; i < 8; i++) pg[i] = pf[0];
+    }
+
     while (cc.valid) {
         const int h0 = (cc.width + 1) >> 1;
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
 #define QUEST_BIG_TILE(NA) \
-    big_tile<OUT, NA>(lds, ld, sg, out, act_rs, wgt_rs, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, vec_par)
+    big_tile<OUT, NA>(lds, ld, ldr, pp, pf, pg, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
         switch (na) {
             case 4: QUEST_BIG_TILE(4); break;
             case 3: QUEST_BIG_TILE(3); break;
@@ -865,9 +910,9 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
             default: QUEST_BIG_TILE(0); break;
         }
 #undef QUEST_BIG_TILE
-        vec_par ^= 1;
         cursor_next_tile(cc);
     }
+    wait_vmcnt_imm<0>();                         // no direct-to-LDS load may outlive the workgroup's LDS allocation
 }
 
 }  // namespace big
@@ -917,7 +962,9 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    if ((K & 255) == 0 && M > 64) return gemm_launch_big<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    // the large-tile kernel fetches b_mul two channels per dword: even N and a 4-byte aligned vector
+    if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && aligned(b_mul, 4))
+        return gemm_launch_big<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
