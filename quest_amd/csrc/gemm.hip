@@ -512,7 +512,8 @@ constexpr int kEpiStride = 136;               // bytes per token row of the epil
 constexpr int kEpiWaveB = 32 * kEpiStride;
 constexpr int kEpiOff = kStages * kStageB;
 constexpr int kVecOff = kEpiOff + 4 * kEpiWaveB;
-constexpr int kVecB = 2 * (kRows * 4 + kRows * 2);   // two parities of (b_add int32, b_mul 16-bit) per channel
+constexpr int kVecParB = 2 * (kRows * 4 + kRows * 2);   // b_add, b_mul per channel and a_add, a_mul per token of one tile
+constexpr int kVecB = 2 * kVecParB;                       // two tiles in flight
 constexpr int kLdsB = kVecOff + kVecB;        // ~148 KiB of the CU's 160 KiB
 
 // s_barrier alone: waves order their own LDS traffic with s_waitcnt, and a release / acquire fence here would
@@ -548,7 +549,7 @@ __device__ __forceinline__ void cursor_next_tile(Cursor &c) {
 }
 
 struct Loader {          // direct-to-LDS loads of one wave: 4 instructions of 16 token rows, 4 of 16 channel rows
-    __amdgpu_buffer_rsrc_t act, wgt, badd, bmul;
+    __amdgpu_buffer_rsrc_t act, wgt, badd, bmul, aadd, amul;
     uint32_t off_t, off_c;      // byte offset of this lane's first row of the load cursor's tile (+ its 16-byte chunk)
     int kbytes, nk, wave;
     int issued;                 // stages issued so far by this workgroup (slot = issued % kStages)
@@ -593,11 +594,11 @@ __device__ __forceinline__ void wait_vmcnt_imm() {
 __device__ __forceinline__ void wait_stage(int extra) {
     constexpr int kBase = kLoads * (kStages - 3);
     switch (extra) {
-        case 34: wait_vmcnt_imm<kBase + 34>(); break;
-        case 26: wait_vmcnt_imm<kBase + 26>(); break;
-        case 18: wait_vmcnt_imm<kBase + 18>(); break;
-        case 10: wait_vmcnt_imm<kBase + 10>(); break;
-        case 2: wait_vmcnt_imm<kBase + 2>(); break;
+        case 36: wait_vmcnt_imm<kBase + 36>(); break;
+        case 28: wait_vmcnt_imm<kBase + 28>(); break;
+        case 20: wait_vmcnt_imm<kBase + 20>(); break;
+        case 12: wait_vmcnt_imm<kBase + 12>(); break;
+        case 4: wait_vmcnt_imm<kBase + 4>(); break;
         default: wait_vmcnt_imm<kBase>(); break;
     }
 }
@@ -648,18 +649,28 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
 
-    // per-channel epilogue vectors of this tile -> LDS, also by direct loads (two per wave: its 64 channels
-    // of b_add and of b_mul); they are read back after the K loop.  Counted in pp.store_extra below.
-    int32_t *v_add = reinterpret_cast<int32_t *>(lds + kVecOff + pp.vec_par * (kRows * 6));
-    uint16_t *v_mul = reinterpret_cast<uint16_t *>(lds + kVecOff + pp.vec_par * (kRows * 6) + kRows * 4);
+    // epilogue vectors of this tile -> LDS, also by direct loads: wave w brings 64 channels of b_add and b_mul
+    // and 64 tokens of a_add and a_mul (four loads per wave, counted in pp.store_extra); read back after the K loop
+    uint8_t *vec = lds + kVecOff + pp.vec_par * kVecParB;
+    int32_t *v_add = reinterpret_cast<int32_t *>(vec);
+    uint16_t *v_mul = reinterpret_cast<uint16_t *>(vec + kRows * 4);
+    int32_t *w_add = reinterpret_cast<int32_t *>(vec + kRows * 6);
+    uint16_t *w_mul = reinterpret_cast<uint16_t *>(vec + kRows * 10);
     if constexpr (OUT != OUT_INT32) {
-        const int c = ch0 + wave * 64 + lane;
+        // a direct load places lane l's data at 4 l bytes whatever its size, so the 16-bit vectors travel as
+        // 32 dwords of two elements
+        const int c = ch0 + wave * 64;
+        const int t = tok0 + wave * 64;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ldr.badd, (__attribute__((address_space(3))) void *)(v_add + wave * 64), 4,
-                                                 c * 4, 0, 0, 0);
-        // a direct load places lane l's data at 4 l bytes whatever its size, so b_mul travels as 32 dwords of two
-        if (lane < 32)
+                                                 (c + lane) * 4, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ldr.aadd, (__attribute__((address_space(3))) void *)(w_add + wave * 64), 4,
+                                                 (t + lane) * 4, 0, 0, 0);
+        if (lane < 32) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ldr.bmul, (__attribute__((address_space(3))) void *)(v_mul + wave * 64), 4,
-                                                     (ch0 + wave * 64 + 2 * lane) * 2, 0, 0, 0);
+                                                     (c + 2 * lane) * 2, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ldr.amul, (__attribute__((address_space(3))) void *)(w_mul + wave * 64), 4,
+                                                     (t + 2 * lane) * 2, 0, 0, 0);
+        }
     }
 
     // packed operand fragments of one k-pair: pf[0..3] the four token sub-tiles, pf[4..] the channel sub-tiles
@@ -720,13 +731,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         uint8_t *ebuf = lds + kEpiOff + wave * kEpiWaveB;
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            const int tok_w = tok0 + wt * 128 + b * 32 + li;      // the token whose values this lane converts
-            int t_add = 0;
+            int t_add = 0;                                         // of the token whose values this lane converts
             float t_half_mul = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                const int tc = tok_w < M ? tok_w : M - 1;
-                t_add = a_add[tc];
-                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(a_mul[tc]));
+                t_add = w_add[wt * 128 + b * 32 + li];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li]));
             }
 #pragma unroll
             for (int a0 = 0; a0 < NA; a0 += kApp) {
@@ -788,8 +797,8 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             int t_add = 0;
             float t_half_mul = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                t_add = a_add[tok];
-                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(a_mul[tok]));
+                t_add = w_add[wt * 128 + b * 32 + li];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li]));
             }
 #pragma unroll
             for (int a = 0; a < NA; a++) {
@@ -816,9 +825,9 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     }
     // how many of this wave's stores the next stage synchronisations may leave in flight: exact only when every
     // store instruction of the fast path was issued with all its lanes (an interior tile), otherwise none
-    // (the next tile's two vector loads, issued right after this point, are always exact)
+    // (the next tile's four vector loads, issued right after this point, are always exact)
     if constexpr (OUT != OUT_INT32) {
-        pp.store_extra = (interior ? 8 * NA : 0) + 2;
+        pp.store_extra = (interior ? 8 * NA : 0) + 4;
         pp.store_syncs = kStages - 2;
     } else {
         pp.store_extra = 0;
@@ -868,6 +877,8 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     ldr.wgt = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, N * kbytes, 0x00020000);
     ldr.badd = __builtin_amdgcn_make_buffer_rsrc((void *)b_add, 0, N * 4, 0x00020000);
     ldr.bmul = __builtin_amdgcn_make_buffer_rsrc((void *)b_mul, 0, N * 2, 0x00020000);
+    ldr.aadd = __builtin_amdgcn_make_buffer_rsrc((void *)a_add, 0, M * 4, 0x00020000);
+    ldr.amul = __builtin_amdgcn_make_buffer_rsrc((void *)a_mul, 0, M * 2, 0x00020000);
     ldr.kbytes = kbytes;
     ldr.nk = K / 128;
     ldr.wave = wave;
@@ -881,7 +892,7 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     plain_barrier();
     Pipe pp;
     pp.it = 0;
-    pp.store_extra = OUT != OUT_INT32 ? 2 : 0;   // the first tile's two vector loads
+    pp.store_extra = OUT != OUT_INT32 ? 4 : 0;   // the first tile's four vector loads
     pp.store_syncs = OUT != OUT_INT32 ? kStages - 2 : 0;
     pp.vec_par = 0;
     v4i pf[8], pg[8];
@@ -962,8 +973,8 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    // the large-tile kernel fetches b_mul two channels per dword: even N and a 4-byte aligned vector
-    if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && aligned(b_mul, 4))
+    // the large-tile kernel fetches the 16-bit scale vectors two per dword: even M, N and 4-byte aligned vectors
+    if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && (M & 1) == 0 && aligned(b_mul, 4) && aligned(a_mul, 4))
         return gemm_launch_big<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
