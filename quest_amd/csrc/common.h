@@ -126,14 +126,29 @@ __device__ __forceinline__ float scale_from_sumsq(float sumsq, int k) {
     return __fadd_rn(__fmul_rn(sd, kGaussInt4Step), kScaleEps);
 }
 
-// clamp(floor(x / s), -8, 7) with an IEEE-correct divide; NaN quotients (0/0) land on -8 like
-// fmaxf/fminf in the CUDA kernel this replaces.
+// clamp(floor(x / s), -8, 7), bit-identical to the IEEE-divide form for 16-bit-float x and s.
+// With inv = fl(1 / s) the product t = fl(x * inv) is within 2^-23 (relative) of x / s.  A quotient of
+// two such numbers that is not an integer lies at least 2^-14 (relative) away from the next one, so
+// only exact-integer quotients can land on the wrong side of their floor; nudging t by 2^-21 |t|
+// towards +inf puts those back (and moves nothing else across an integer).  NaN (0 / 0) comes out
+// of v_med3_f32 as -8, like fmaxf / fminf in the CUDA kernel this replaces.
+__device__ __forceinline__ float quant_inv(float s) { return __fdiv_rn(1.0f, s); }
+__device__ __forceinline__ float quant_code_inv(float x, float inv) {
+    const float t = __fmul_rn(x, inv);
+    const float tn = __builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t);      // 2^-21
+    return __builtin_floorf(__builtin_amdgcn_fmed3f(tn, -8.f, 7.5f));
+}
+// reference form with the correctly rounded divide (kept for the exhaustive equivalence test)
 __device__ __forceinline__ float quant_code(float x, float s) {
     float q = __builtin_floorf(__fdiv_rn(x, s));
     q = fmaxf(q, -8.f);
     q = fminf(q, 7.f);
     return q;
 }
+
+// hadamard_mfma.hip: the matrix-core fused activation kernel; QUEST_ERR_UNSUPPORTED when it does not apply
+int launch_hadamard_quantize_mfma(const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had, int K,
+                                  int M, float had_scale, int dtype, hipStream_t st);
 
 inline int check_dtype(int dtype) { return dtype == QUEST_DTYPE_BF16 || dtype == QUEST_DTYPE_FP16; }
 inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

@@ -131,12 +131,13 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
     const float s = to_f32<DT>(s16);
 
     if (packed == nullptr && row_sum == nullptr) return;
+    const float inv = quant_inv(s);
     int isum = 0;
 #pragma unroll
     for (int i = 0; i < NCHUNK; i++) {
         float q[8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = quant_code(y[i][e], s);
+        for (int e = 0; e < 8; e++) q[e] = quant_code_inv(y[i][e], inv);
         int csum = 0;
         const uint32_t w = pack_nibbles8(q, csum);
         const int c = i * BLOCK + tid;
@@ -204,12 +205,13 @@ quantize_kernel(uint16_t *__restrict__ x, const uint16_t *__restrict__ scale, in
     uint4 *xr = reinterpret_cast<uint4 *>(x + (size_t)row * K);
     const float s = to_f32<DT>(scale[row]);
     const float half_s = __fmul_rn(s, 0.5f);
+    const float inv = quant_inv(s);
     int isum = 0;
     for (int c = threadIdx.x; c < nchunks; c += 256) {
         float v[8], q[8];
         unpack8<DT>(xr[c], v);
 #pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = quant_code(v[e], s);
+        for (int e = 0; e < 8; e++) q[e] = quant_code_inv(v[e], inv);
         if (do_dequantize) {
 #pragma unroll
             for (int e = 0; e < 8; e++) v[e] = __fadd_rn(__fmul_rn(q[e], s), half_s);
@@ -348,6 +350,10 @@ extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t 
     if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
     if (!aligned(x, 16) || !aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
     hipStream_t st = (hipStream_t)stream;
+    // rows of up to 4096 with the activation transform: Hadamard on the matrix cores; anything else: butterflies
+    const int rc = launch_hadamard_quantize_mfma(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size,
+                                                 had_scale, dtype, st);
+    if (rc != QUEST_ERR_UNSUPPORTED) return rc;
     if (dtype == QUEST_DTYPE_BF16)
         return launch_hadamard_quantize<0>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale, st);
     return launch_hadamard_quantize<1>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale, st);
