@@ -47,6 +47,20 @@ template <int DT>
 __device__ __forceinline__ uint32_t pack2_from_f32(float lo, float hi) {
     return from_f32<DT>(lo) | (from_f32<DT>(hi) << 16);
 }
+// The same pair as one two-element conversion (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32, both round to
+// nearest even).  Only for values that do not come out of an fp32 multiply (see from_f32).
+template <int DT>
+__device__ __forceinline__ uint32_t pack2_rne(float lo, float hi) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    if constexpr (DT == QUEST_DTYPE_BF16) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+    } else {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    }
+}
 
 // ---- cross-lane moves -----------------------------------------------------------------------
 // value of lane (lane ^ M); M = 1, 2, 8 are single DPP moves, 4 and 16 LDS-crossbar swizzles.
@@ -82,6 +96,29 @@ __device__ __forceinline__ int wave_sum_i(int v) {
     v += lane_xor_i<16>(v);
     v += lane_xor_i<32>(v);
     return v;
+}
+
+// Sum over the 64 lanes with DPP moves only (no LDS crossbar traffic); lane 0..63 all get the total.
+// Pairing inside 16 lanes: xor 1, xor 2, mirror of 8 (any pairing serves a symmetric sum), rotate by 8;
+// then the four 16-lane totals are read as scalars and added in lane order.
+__device__ __forceinline__ float wave_sum_dpp_f(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));   // row_ror:8
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return ((a + b) + c) + d;
+}
+__device__ __forceinline__ int wave_sum_dpp_i(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true);
+    return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+           __builtin_amdgcn_readlane(v, 48);
 }
 
 // Block all-reduce through LDS: per-wave totals are added in wave order by every thread.
@@ -137,6 +174,15 @@ __device__ __forceinline__ float quant_code_inv(float x, float inv) {
     const float t = __fmul_rn(x, inv);
     const float tn = __builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t);      // 2^-21
     return __builtin_floorf(__builtin_amdgcn_fmed3f(tn, -8.f, 7.5f));
+}
+// the same code as an integer: the clamp makes the floor-and-convert instruction safe
+__device__ __forceinline__ int quant_code_inv_i(float x, float inv) {
+    const float t = __fmul_rn(x, inv);
+    const float tn = __builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t);
+    const float m = __builtin_amdgcn_fmed3f(tn, -8.f, 7.5f);
+    int q;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(m));
+    return q;
 }
 // reference form with the correctly rounded divide (kept for the exhaustive equivalence test)
 __device__ __forceinline__ float quant_code(float x, float s) {

@@ -350,7 +350,7 @@ extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t 
     if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
     if (!aligned(x, 16) || !aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
     hipStream_t st = (hipStream_t)stream;
-    // rows of up to 4096 with the activation transform: Hadamard on the matrix cores; anything else: butterflies
+    // rows of up to 32768 with a Hadamard entry the dtype holds exactly: matrix cores; anything else: butterflies
     const int rc = launch_hadamard_quantize_mfma(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size,
                                                  had_scale, dtype, st);
     if (rc != QUEST_ERR_UNSUPPORTED) return rc;

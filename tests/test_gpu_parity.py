@@ -202,10 +202,11 @@ def test_hadamard128(quest, dtype, scale):
 # --------------------------------------------------------------------------- fused activation kernel
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768), (64, 4096), (1, 128), (8, 11008), (16, 2816), (2, 16384), (2, 32768),
-                                   (3, 1024), (777, 4096), (5, 3968)])
+                                   (3, 1024), (777, 4096), (5, 3968), (3, 5120), (6, 8192), (2, 28672), (2, 65536)])
 def test_hadamard_quantize_fused(quest, dtype, shape):
-    """Rows of up to 4096 run the Hadamard on the matrix cores (the reference's matmul formulation, fp32
-    accumulation in the hardware's order), longer rows run fp32 butterflies."""
+    """Rows of up to 32768 run the Hadamard on the matrix cores (the reference's matmul formulation, fp32
+    accumulation in the hardware's order; rows over 4096 are shared by the waves of a workgroup), longer
+    rows run fp32 butterflies."""
     m, k = shape
     x = rand_act(m, k, dtype, seed=10)
     gx = x.to(DEV)
@@ -219,7 +220,7 @@ def test_hadamard_quantize_fused(quest, dtype, shape):
         assert ((had.double() - ref.double()).norm() / ref.double().norm()) < 1e-3
         tol = ref.double().abs().amax(-1, keepdim=True) * 2. ** -8
         assert ((had.double() - ref.double()).abs() <= tol).all()
-    if k > 4096:
+    if k > 32768:
         assert torch.equal(bits(had), bits(qo.hadamard128_fwht(x, 181. / 2048.)))      # butterfly kernel: same order, same bits
     # (2) scale on the kernel's own transformed tensor: within one ulp of the oracle, rarely different
     want_scale = qo.find_scale_int4(had)
@@ -241,6 +242,23 @@ def test_hadamard_quantize_fused(quest, dtype, shape):
     # (5) outputs that are not asked for are not needed: scale only, and codes without the debug tensor
     s3, p3, r3 = quest.hadamard_quantize_int4(gx)
     assert torch.equal(bits(s3.cpu()), bits(scale.cpu())) and torch.equal(p3, packed) and torch.equal(r3, row_sum)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_hadamard_quantize_weight_scale_runs_butterflies(quest, dtype):
+    """2^-3.5 (the weight-side factor) is not a 16-bit float, so the fused kernel keeps fp32 butterflies and an
+    fp32 factor: same bits as the butterfly oracle, and the fused codes equal the composition of the steps."""
+    w = rand_act(96, 2048, dtype, seed=13)
+    gw = w.to(DEV)
+    w_had = torch.empty_like(gw)
+    scale, packed, row_sum = quest.hadamard_quantize_int4(gw, x_had=w_had, hadamard_scale=2. ** -3.5)
+    want_had = qo.hadamard128_fwht(w, 2. ** -3.5)
+    assert torch.equal(bits(w_had.cpu()), bits(want_had))
+    assert ulp_diff(scale, qo.find_scale_int4(want_had)).max() <= 1
+    xp = torch.empty(96, 1024, dtype=torch.uint8)
+    rs = torch.empty(96, 1, dtype=torch.int32)
+    qo.quantize_int4(want_had.clone(), scale.cpu(), None, xp, rs, False)
+    assert torch.equal(packed.cpu(), xp) and torch.equal(row_sum.cpu(), rs)
 
 
 def test_hadamard_quantize_is_deterministic(quest):
