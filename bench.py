@@ -9,7 +9,7 @@ INT4 x INT4 GEMM with the scale epilogue to fp16.  Inputs are synthetic and alre
 HBM; several activation buffers are rotated so that no step finds its input in the Infinity Cache.
 `value` is 2*M*N*K / step time (TOPS of the whole linear, as the reference's published layer times
 are converted).  The JSON line also carries
-  roofline           the GEMM kernel against the INT8 MFMA peak (HIP-event time per launch),
+  roofline           the GEMM kernel against the INT8 MFMA peak (HIP events around back-to-back launches),
   roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
                      outlier channels) against the HBM peak,
   decode             the GEMM at M in {1, 8, 16}, weight streaming,
@@ -32,10 +32,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 INT8_MFMA_PEAK_TOPS = 5000.0
 
-# HBM bytes per launch read from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), scaled by a copy
-# kernel of known size; None until such a run has been recorded under profiles/.
-TRAFFIC_GEMM_BYTES = None
-TRAFFIC_QUANTIZE_BYTES = None
+# HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
+# scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.99979, WRITE_SIZE x 1.0);
+# the runs are summarised under profiles/.
+TRAFFIC_GEMM_BYTES = int((128273.8 * 1.99979 + 109677.0) * 1024)        # M=4096 K=4096 N=11008 fp16
+TRAFFIC_QUANTIZE_BYTES = int((32814.8 * 1.99979 + 16512.9) * 1024)      # bf16 [8192, 4096]
 
 
 def event_pairs(n):
@@ -44,6 +45,22 @@ def event_pairs(n):
 
 def mean_ms(pairs):
     return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+
+
+def launches_ms(launch, n, warmup=5):
+    """Average duration of `n` back-to-back launches of one kernel: HIP events on torch's current stream (the
+    stream the launches are given) around the whole batch.  `launch(i)` must be a bare C-ABI call, cheap enough
+    on the host that the queue never runs dry; gaps between kernels count as kernel time."""
+    for i in range(warmup):
+        launch(i)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for i in range(n):
+        launch(i)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / n
 
 
 def heavy_tailed_activations(m, k, dtype, device, seed):
@@ -57,7 +74,7 @@ def heavy_tailed_activations(m, k, dtype, device, seed):
     return x.to(dtype).to(device)
 
 
-def bench_linear(quest, harness, steps, warmup, dev):
+def bench_linear(quest, _lib, steps, warmup, dev):
     m, k, n = 4096, 4096, 11008
     dtype = torch.float16
     g = torch.Generator(device='cpu').manual_seed(0)
@@ -94,7 +111,19 @@ def bench_linear(quest, harness, steps, warmup, dev):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
     quant_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
-    gemm_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    gemm_in_step_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+
+    # the GEMM alone, bare C-ABI launches on the codes the last step left
+    lib = _lib.load()
+    st = _lib.stream_of(out)
+    args = (_lib.ptr(out), _lib.ptr(a_packed), _lib.ptr(w_packed), _lib.ptr(a_row_sum), _lib.ptr(w_add),
+            _lib.ptr(a_scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype], st)       # sizes in the ABI's order: M, K, N
+
+    def gemm(_):
+        if lib.quest_fused_matmul_dequantize_int4_int4t(*args) != 0:
+            raise RuntimeError('GEMM launch failed')
+
+    gemm_ms = launches_ms(gemm, max(steps, 20))
     ops = 2.0 * m * n * k
     return {
         'shape': {'M': m, 'K': k, 'N': n},
@@ -102,11 +131,12 @@ def bench_linear(quest, harness, steps, warmup, dev):
         'tops': ops / (ms_per_step * 1e-3) / 1e12,
         'gemm_ms': gemm_ms,
         'gemm_tops': ops / (gemm_ms * 1e-3) / 1e12,
+        'gemm_in_step_ms': gemm_in_step_ms,
         'quant_ms': quant_ms,
     }
 
 
-def bench_quantize(quest, steps, warmup, dev):
+def bench_quantize(_lib, steps, warmup, dev):
     m, k = 8192, 4096
     dtype = torch.bfloat16
     n_buf = 6                                   # 6 x 64 MiB > the 256 MB Infinity Cache
@@ -114,20 +144,20 @@ def bench_quantize(quest, steps, warmup, dev):
     scale = torch.empty(m, 1, dtype=dtype, device=dev)
     packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
     row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
-    for i in range(warmup):
-        quest.hadamard_quantize_int4(xs[i % n_buf], scale, packed, row_sum)
-    pairs = event_pairs(steps)
-    torch.cuda.synchronize()
-    for i, (a, b) in enumerate(pairs):
-        a.record()
-        quest.hadamard_quantize_int4(xs[i % n_buf], scale, packed, row_sum)
-        b.record()
-    torch.cuda.synchronize()
-    ms = mean_ms(pairs)
+    lib = _lib.load()
+    st = _lib.stream_of(scale)
+    xp = [_lib.ptr(x) for x in xs]
+    tail = (_lib.ptr(scale), _lib.ptr(packed), _lib.ptr(row_sum), None, k, m, 181. / 2048., _lib.DTYPE_CODE[dtype], st)
+
+    def launch(i):
+        if lib.quest_hadamard_quantize_int4(xp[i % n_buf], *tail) != 0:
+            raise RuntimeError('activation kernel launch failed')
+
+    ms = launches_ms(launch, steps, warmup)
     algo_bytes = m * k * 2 + m * k // 2 + m * 2 + m * 4
     gbs = algo_bytes / (ms * 1e-3) / 1e9
     return {'bound': 'hbm', 'achieved': gbs, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs / HBM_PEAK_GBS,
-            'traffic': TRAFFIC_QUANTIZE_BYTES, 'kernel': 'hadamard_quantize_kernel', 'us_per_launch': ms * 1e3,
+            'traffic': TRAFFIC_QUANTIZE_BYTES, 'kernel': 'hadamard_quantize_mfma_kernel', 'us_per_launch': ms * 1e3,
             'algorithmic_bytes': algo_bytes, 'workload': 'bf16 [8192,4096] Student-t(3), 1% channels x20'}
 
 
@@ -203,6 +233,16 @@ def bench_cpu_baseline():
                                'value': ops / t32[len(t32) // 2] / 1e12, 'ms_per_call': t32[len(t32) // 2] * 1e3}}
 
 
+def calibration_stream(dev):
+    """A plain elementwise kernel of known traffic (reads 256 MiB, writes 256 MiB), launched three times so that
+    a counter run of this script holds the reference the FETCH_SIZE / WRITE_SIZE readings are scaled by."""
+    a = torch.zeros(64 * 1024 * 1024, dtype=torch.int32, device=dev)
+    b = torch.empty_like(a)
+    for _ in range(3):
+        torch.add(a, 1, out=b)
+    torch.cuda.synchronize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -216,19 +256,20 @@ def main():
     if not torch.cuda.is_available():
         sys.exit('bench.py: no GPU visible')
     import quest_amd as quest
-    from quest_amd import _lib, harness
+    from quest_amd import _lib
     _lib.load()
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
 
-    lin = bench_linear(quest, harness, args.steps, args.warmup, dev)
-    rq = bench_quantize(quest, max(args.steps, 20), args.warmup, dev)
+    lin = bench_linear(quest, _lib, args.steps, args.warmup, dev)
+    rq = bench_quantize(_lib, max(args.steps, 60), args.warmup, dev)
     dec = bench_decode(quest, dev)
+    calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
 
     roofline = {'bound': 'mfma', 'achieved': lin['gemm_tops'], 'peak': INT8_MFMA_PEAK_TOPS, 'unit': 'TOP/s',
                 'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES,
-                'kernel': 'gemm_w4a4_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
+                'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
                 'algorithmic_ops': 2.0 * 4096 * 4096 * 11008}
     line = {
         'metric': 'INT4-GEMM TOPS + quantize GB/s at Llama-7B layer shapes, % MI355X roofline',
@@ -238,7 +279,8 @@ def main():
         'config': {'workload': 'W4A4 linear, Llama-7B gate/up: fp16 activations [4096,4096] -> fused '
                                'Hadamard-quantize-pack -> packed INT4 GEMM [4096,4096]x[11008,4096]^T -> fp16 [4096,11008]',
                    'M': 4096, 'K': 4096, 'N': 11008},
-        'gemm_tops': lin['gemm_tops'], 'quantize_us_in_step': lin['quant_ms'] * 1e3,
+        'gemm_tops': lin['gemm_tops'], 'gemm_us_in_step': lin['gemm_in_step_ms'] * 1e3,
+        'quantize_us_in_step': lin['quant_ms'] * 1e3,
         'quantize_GBs': rq['achieved'],
         'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'cpu_baseline': cpu,
     }
