@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 LIB_PATH = os.path.join(HERE, 'libquest_hip.so')
-SOURCES = ['rowops.hip', 'hadamard_mfma.hip', 'gemm.hip', 'capi.hip']
+SOURCES = ['rowops.hip', 'hadamard_mfma.hip', 'gemm.hip', 'gemm_decode.hip', 'capi.hip']
 
 FLAGS = [
     '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-shared',

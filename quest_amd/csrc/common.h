@@ -192,6 +192,13 @@ __device__ __forceinline__ float quant_code(float x, float s) {
     return q;
 }
 
+// what a GEMM writes: the two 16-bit float types share their codes with QUEST_DTYPE_*
+enum { OUT_BF16 = 0, OUT_FP16 = 1, OUT_INT32 = 2 };
+
+// gemm_decode.hip: the weight-streaming GEMM for M <= 64; QUEST_ERR_UNSUPPORTED when it does not apply
+int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                       const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);
+
 // hadamard_mfma.hip: the matrix-core fused activation kernel; QUEST_ERR_UNSUPPORTED when it does not apply
 int launch_hadamard_quantize_mfma(const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had, int K,
                                   int M, float had_scale, int dtype, hipStream_t st);

@@ -33,8 +33,6 @@ constexpr int kTileBytes = kTileRows * kRowBytes;    // 32 KiB
 constexpr int kStageBytes = 2 * kTileBytes;          // channel tile + token tile
 constexpr int kLdsBytes = 2 * kStageBytes;           // double buffered: 128 KiB of the CU's 160 KiB
 
-enum { OUT_BF16 = 0, OUT_FP16 = 1, OUT_INT32 = 2 };
-
 __device__ __forceinline__ void lds_fence_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
@@ -973,6 +971,11 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    // a handful of tokens: the weight-streaming kernel
+    if (M <= 64) {
+        const int rc = launch_gemm_decode(OUT, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        if (rc != QUEST_ERR_UNSUPPORTED) return rc;
+    }
     // the large-tile kernel fetches the 16-bit scale vectors two per dword: even M, N and 4-byte aligned vectors
     if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && (M & 1) == 0 && aligned(b_mul, 4) && aligned(a_mul, 4))
         return gemm_launch_big<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);

@@ -1,0 +1,183 @@
+// Packed-INT4 x packed-INT4 GEMM for a handful of tokens (M <= 64): the weight matrix is streamed
+// from HBM exactly once and that stream is the whole cost, so the kernel is laid out around it.
+//
+// Same arithmetic and outputs as the large GEMM (gemm-quest/quest/matmul_kernel.cu:8-63 and
+// gemm-quest/quest/fused_matmul_dequantize_kernel.cu:4-57 of the reference, which run their one
+// CUTLASS tile shape at every M); this is the shape the reference's decode benchmark exercises
+// (gemm-quest/benchmarks/bench_e2e.py with one token per sequence).
+//
+// A workgroup of eight waves owns 16 output channels over the whole K; wave w takes the 256-k
+// chunks w, w + 8, ...  For a chunk a lane (r = lane % 16, g = lane / 16) loads two 16-byte pieces
+// of weight row r -- bytes 16 g and 64 + 16 g of the chunk's 128 -- so the wave's two loads cover one
+// whole 128-byte line of each of its 16 rows, and the same two pieces of token row r.  A piece is 32
+// nibbles: `w & 0xF0F0F0F0` is 16 * (odd-k nibbles), `(w << 4) & 0xF0F0F0F0` is 16 * (even-k
+// nibbles), both sign-correct int8, each feeding one v_mfma_i32_16x16x64_i8 (weights as the "A"
+// operand, tokens as "B"; both operands permute k identically, which a dot product ignores).  All
+// of a wave's loads for up to four chunks are in flight before the first is used.  The eight partial
+// 16 x 16 tiles meet in LDS, the factor 256 the nibble trick leaves is shifted out exactly, and the
+// first wave(s) apply the scale epilogue and store four consecutive channels of a token per lane.
+#include "common.h"
+
+namespace quest {
+namespace decode {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 8;
+constexpr int kChannels = 16;             // output channels per workgroup
+constexpr int kChunkB = 128;              // packed bytes per row per chunk (256 k)
+constexpr int kBatch = 4;                 // chunks whose loads are in flight together
+
+__device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        odd[d] = p[d] & (int)0xF0F0F0F0u;
+        even[d] = (p[d] << 4) & (int)0xF0F0F0F0u;
+    }
+}
+
+// TM = token tiles of 16 (M <= 16 TM)
+template <int OUT, int TM>
+__global__ void __launch_bounds__(64 * kWaves)
+gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
+                        const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
+                        const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul, int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) int red[kWaves][TM][64][4];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int row_b = K >> 1;                          // packed bytes per row
+    const int ch0 = blockIdx.x * kChannels;
+    const int n_chunks = (row_b + kChunkB - 1) / kChunkB;      // the last one may hold only its first 64 bytes
+
+    // rows that do not exist get an offset beyond the buffer: such loads touch no memory and return zeros
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, (int)((long)N * row_b), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ar = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, (int)((long)M * row_b), 0x00020000);
+    const uint32_t dead = 0x80000000u;                 // buffers are smaller than 2^31 bytes; sums below stay under 2^32
+    const uint32_t w_off = (ch0 + r < N) ? (uint32_t)((ch0 + r) * row_b + g * 16) : dead;
+    uint32_t a_off[TM];
+#pragma unroll
+    for (int t = 0; t < TM; t++) a_off[t] = (t * 16 + r < M) ? (uint32_t)((t * 16 + r) * row_b + g * 16) : dead;
+
+    v4i acc[TM];
+#pragma unroll
+    for (int t = 0; t < TM; t++) acc[t] = v4i{0, 0, 0, 0};
+
+    for (int c0 = wave; c0 < n_chunks; c0 += kWaves * kBatch) {
+        v4i wq[kBatch][2], aq[kBatch][TM][2];
+#pragma unroll
+        for (int i = 0; i < kBatch; i++) {
+            const int c = c0 + i * kWaves;
+            const int cb = c * kChunkB;
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                // a piece past the end of the row (chunk index too large, or the second half of a 64-byte tail) reads as zero
+                const bool in_row = c < n_chunks && cb + 64 * hlf < row_b;
+                const uint32_t shift = (uint32_t)(cb + 64 * hlf);
+                wq[i][hlf] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, (int)(in_row ? w_off + shift : dead), 0, 0));
+#pragma unroll
+                for (int t = 0; t < TM; t++)
+                    aq[i][t][hlf] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, (int)(in_row ? a_off[t] + shift : dead), 0, 0));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; i++)
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                v4i we, wo;
+                split16(wq[i][hlf], we, wo);
+#pragma unroll
+                for (int t = 0; t < TM; t++) {
+                    v4i ae, ao;
+                    split16(aq[i][t][hlf], ae, ao);
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(we, ae, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wo, ao, acc[t], 0, 0, 0);
+                }
+            }
+    }
+
+    // ---- partial tiles meet in LDS
+#pragma unroll
+    for (int t = 0; t < TM; t++) *reinterpret_cast<v4i *>(&red[wave][t][lane][0]) = acc[t];
+    __syncthreads();
+    if (wave >= TM) return;
+    const int t = wave;                                  // wave t finishes token tile t
+    v4i sum = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) {
+        const v4i p = *reinterpret_cast<const v4i *>(&red[w][t][lane][0]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum[e] += p[e];
+    }
+
+    // ---- lane (r, g) holds channels ch0 + 4 g + {0..3} of token 16 t + r
+    const int tok = t * 16 + r;
+    const int ch = ch0 + 4 * g;
+    if (tok >= M || ch >= N) return;
+    int c[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) c[e] = sum[e] >> 8;      // exact: every product carries 16 * 16
+    const size_t o = (size_t)tok * N + ch;
+    if constexpr (OUT == OUT_INT32) {
+        int32_t *dst = reinterpret_cast<int32_t *>(out) + o;
+        if ((N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+            *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (ch + e < N) dst[e] = c[e];
+        }
+    } else {
+        const int t_add = a_add[tok];
+        const float t_half_mul = __fmul_rn(0.5f, to_f32<OUT>(a_mul[tok]));
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int che = (ch + e < N) ? ch + e : N - 1;
+            const float lhs = (float)(c[e] * 2 + t_add + b_add[che]);
+            const float rhs = __fmul_rn(t_half_mul, to_f32<OUT>(b_mul[che]));
+            h[e] = from_f32<OUT>(__fmul_rn(lhs, rhs));
+        }
+        uint16_t *dst = reinterpret_cast<uint16_t *>(out) + o;
+        if ((N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0) {
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (ch + e < N) dst[e] = (uint16_t)h[e];
+        }
+    }
+}
+
+template <int OUT, int TM>
+static void launch_tm(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
+                      const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    gemm_w4a4_decode_kernel<OUT, TM><<<dim3((N + kChannels - 1) / kChannels), dim3(64 * kWaves), 0, st>>>(
+        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K);
+}
+
+template <int OUT>
+static int launch_out(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
+                      const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    if (M <= 16) launch_tm<OUT, 1>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    else if (M <= 32) launch_tm<OUT, 2>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    else launch_tm<OUT, 4>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    return launch_status();
+}
+
+}  // namespace decode
+
+// The weight-streaming kernel applies to M <= 64 and K a multiple of 128 (whole 64-byte pieces); QUEST_ERR_UNSUPPORTED otherwise.
+int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                       const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    if (M > 64 || (K & 127) != 0 || !aligned(a, 16) || !aligned(b, 16)) return QUEST_ERR_UNSUPPORTED;
+    switch (out_kind) {
+        case OUT_BF16: return decode::launch_out<OUT_BF16>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        case OUT_FP16: return decode::launch_out<OUT_FP16>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        default: return decode::launch_out<OUT_INT32>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    }
+}
+
+}  // namespace quest
