@@ -12,7 +12,7 @@ are converted).  The JSON line also carries
   roofline           the GEMM kernel against the INT8 MFMA peak (HIP events around back-to-back launches),
   roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
                      outlier channels) against the HBM peak,
-  decode             the GEMM at M in {1, 8, 16}, weight streaming,
+  decode             the layer at M in {1, 8, 16}: the weight-streaming GEMM alone and with the activation kernel,
   cpu_baseline       the CPU oracle (PyTorch restatement of the reference's `backend='pytorch'`
                      path) on the reference's CPU-runnable case, timed on this host's cores.
 """
@@ -161,12 +161,16 @@ def bench_quantize(_lib, steps, warmup, dev):
             'algorithmic_bytes': algo_bytes, 'workload': 'bf16 [8192,4096] Student-t(3), 1% channels x20'}
 
 
-def bench_decode(quest, dev):
+def bench_decode(_lib, dev):
+    """The layer at M in {1, 8, 16}: weights rotate through copies totalling more than the Infinity Cache so that they
+    stream from HBM; bare C-ABI launches, the GEMM alone and the activation kernel + GEMM pair."""
     out = []
+    lib = _lib.load()
     dtype = torch.float16
+    code = _lib.DTYPE_CODE[dtype]
     g = torch.Generator(device='cpu').manual_seed(1)
-    for k, n in [(4096, 4096), (11008, 4096)]:
-        n_w = 8                                  # rotate weight copies so they stream from HBM
+    for k, n in [(4096, 4096), (4096, 11008), (11008, 4096)]:
+        n_w = max(2, int(600e6 // (n * k // 2)))
         ws = [torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.uint8).to(dev) for _ in range(n_w)]
         w_scale = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
         w_add = torch.randint(-500, 500, (n, 1), generator=g, dtype=torch.int32).to(dev)
@@ -176,24 +180,28 @@ def bench_decode(quest, dev):
             a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
             a_row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
             y = torch.empty(m, n, dtype=dtype, device=dev)
+            st = _lib.stream_of(y)
+            q_args = (_lib.ptr(x), _lib.ptr(a_scale), _lib.ptr(a_packed), _lib.ptr(a_row_sum), None, k, m, 181. / 2048., code, st)
+            wp = [_lib.ptr(w) for w in ws]
+            g_tail = (_lib.ptr(a_row_sum), _lib.ptr(w_add), _lib.ptr(a_scale), _lib.ptr(w_scale), m, k, n, code, st)
+            yp, ap = _lib.ptr(y), _lib.ptr(a_packed)
 
-            def run(i):
-                quest.hadamard_quantize_int4(x, a_scale, a_packed, a_row_sum)
-                quest.fused_matmul_dequantize_int4_int4t_bf16(a_packed, ws[i % n_w], a_row_sum, w_add, a_scale, w_scale, y)
+            def gemm(i):
+                if lib.quest_fused_matmul_dequantize_int4_int4t(yp, ap, wp[i % n_w], *g_tail) != 0:
+                    raise RuntimeError('GEMM launch failed')
 
-            for i in range(5):
-                run(i)
-            pairs = event_pairs(40)
-            torch.cuda.synchronize()
-            for i, (a, b) in enumerate(pairs):
-                a.record()
-                run(i)
-                b.record()
-            torch.cuda.synchronize()
-            us = mean_ms(pairs) * 1e3
+            def layer(i):
+                if lib.quest_hadamard_quantize_int4(*q_args) != 0:
+                    raise RuntimeError('activation kernel launch failed')
+                gemm(i)
+
+            layer(0)
+            gemm_us = launches_ms(gemm, 200, 20) * 1e3
+            layer_us = launches_ms(layer, 200, 20) * 1e3
             wbytes = n * k // 2
-            out.append({'M': m, 'K': k, 'N': n, 'us': round(us, 2), 'weight_GBs': round(wbytes / us / 1e3, 1),
-                        'frac_hbm': round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+            out.append({'M': m, 'K': k, 'N': n, 'gemm_us': round(gemm_us, 2), 'layer_us': round(layer_us, 2),
+                        'weight_GBs': round(wbytes / gemm_us / 1e3, 1),
+                        'frac_hbm': round(wbytes / gemm_us / 1e3 / HBM_PEAK_GBS, 4)})
     return out
 
 
@@ -263,7 +271,7 @@ def main():
 
     lin = bench_linear(quest, _lib, args.steps, args.warmup, dev)
     rq = bench_quantize(_lib, max(args.steps, 60), args.warmup, dev)
-    dec = bench_decode(quest, dev)
+    dec = bench_decode(_lib, dev)
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
 

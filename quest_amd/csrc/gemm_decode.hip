@@ -61,6 +61,24 @@ gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
 #pragma unroll
     for (int t = 0; t < TM; t++) a_off[t] = (t * 16 + r < M) ? (uint32_t)((t * 16 + r) * row_b + g * 16) : dead;
 
+    // the waves that will finish a token tile fetch their epilogue operands now, off the critical path
+    // (lane (r, g) of wave t ends up with channels ch0 + 4 g + {0..3} of token 16 t + r)
+    int t_add = 0, c_add[4] = {0, 0, 0, 0};
+    float t_half_mul = 0.f, c_mul[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (OUT != OUT_INT32) {
+        if (wave < TM) {
+            const int tok = min(wave * 16 + r, M - 1);
+            t_add = a_add[tok];
+            t_half_mul = __fmul_rn(0.5f, to_f32<OUT>(a_mul[tok]));
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int che = min(ch0 + 4 * g + e, N - 1);
+                c_add[e] = b_add[che];
+                c_mul[e] = to_f32<OUT>(b_mul[che]);
+            }
+        }
+    }
+
     v4i acc[TM];
 #pragma unroll
     for (int t = 0; t < TM; t++) acc[t] = v4i{0, 0, 0, 0};
@@ -112,7 +130,6 @@ gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
         for (int e = 0; e < 4; e++) sum[e] += p[e];
     }
 
-    // ---- lane (r, g) holds channels ch0 + 4 g + {0..3} of token 16 t + r
     const int tok = t * 16 + r;
     const int ch = ch0 + 4 * g;
     if (tok >= M || ch >= N) return;
@@ -130,14 +147,11 @@ gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
                 if (ch + e < N) dst[e] = c[e];
         }
     } else {
-        const int t_add = a_add[tok];
-        const float t_half_mul = __fmul_rn(0.5f, to_f32<OUT>(a_mul[tok]));
         uint32_t h[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const int che = (ch + e < N) ? ch + e : N - 1;
-            const float lhs = (float)(c[e] * 2 + t_add + b_add[che]);
-            const float rhs = __fmul_rn(t_half_mul, to_f32<OUT>(b_mul[che]));
+            const float lhs = (float)(c[e] * 2 + t_add + c_add[e]);
+            const float rhs = __fmul_rn(t_half_mul, c_mul[e]);
             h[e] = from_f32<OUT>(__fmul_rn(lhs, rhs));
         }
         uint16_t *dst = reinterpret_cast<uint16_t *>(out) + o;
