@@ -616,9 +616,57 @@ __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
     }
 }
 
+// The int8 operands of one k-pair (two MFMA k-steps): 16 * even-k nibbles and 16 * odd-k nibbles of the four token
+// sub-tiles and of up to four channel sub-tiles.
+struct Frags {
+    v4i te[4], to[4], ce[4], co[4];
+};
+
+// One k-pair of the main loop, written as 8 NA slots of one MFMA each with the other work of the pipeline spread
+// between them and the order pinned (a lone wave per SIMD issues in order: VALU work, LDS reads and the stage
+// synchronisation only overlap the matrix pipe if they sit between MFMAs, which are 32 cycles apart):
+//   * the MFMAs of this k-pair, operands in `cur`;
+//   * `sync` runs after slot kSyncSlot (-1: none);
+//   * NEXT: the packed fragments of the next k-pair are read from LDS in the slots after that, up to 3/8 of the
+//     way, and split into `nxt` (3 VALU ops per dword) over the second half of the slots.
+template <int NA, bool NEXT, int kSyncSlot, typename Sync>
+__device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Frags &cur, Frags &nxt, const uint8_t *rd_tok,
+                                       const uint8_t *rd_chn, Sync &&sync) {
+    constexpr int S = 8 * NA;                 // slots
+    constexpr int F = 4 + NA;                 // fragments per k-pair
+    constexpr int V = F * 4;                  // dwords to split
+    constexpr int R0 = kSyncSlot + 1;         // reads go into slots [R0, R1)
+    constexpr int R1 = S * 3 / 8 > R0 ? S * 3 / 8 : R0 + 1;
+    constexpr int U0 = S / 2 > R1 ? S / 2 : R1;      // splitting goes into slots [U0, S)
+    v4i raw[8];
+#pragma unroll
+    for (int i = 0; i < S; i++) {
+        const int a = i >> 3, odd = (i >> 2) & 1, b = i & 3;
+        acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(odd ? cur.co[a] : cur.ce[a], odd ? cur.to[b] : cur.te[b], acc[a][b],
+                                                          0, 0, 0);
+        if (i == kSyncSlot) sync();
+        if constexpr (NEXT) {
+            if (i >= R0 && i < R1) {
+#pragma unroll
+                for (int r = (i - R0) * F / (R1 - R0); r < (i - R0 + 1) * F / (R1 - R0); r++)
+                    raw[r] = *reinterpret_cast<const v4i *>(r < 4 ? rd_tok + r * 32 * kRowB : rd_chn + (r - 4) * 32 * kRowB);
+            }
+            if (i >= U0) {
+#pragma unroll
+                for (int v = (i - U0) * V / (S - U0); v < (i - U0 + 1) * V / (S - U0); v++) {
+                    const int f = v >> 2, d = v & 3;
+                    const uint32_t pk = (uint32_t)raw[f][d];
+                    const int ev = (int)((pk << 4) & 0xF0F0F0F0u), od = (int)(pk & 0xF0F0F0F0u);
+                    if (f < 4) { nxt.te[f][d] = ev; nxt.to[f][d] = od; } else { nxt.ce[f - 4][d] = ev; nxt.co[f - 4][d] = od; }
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 template <int OUT, int NA>
-__device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, v4i (&pf)[8], v4i (&pg)[8],
-                                         void *__restrict__ out, const int32_t *__restrict__ a_add,
+__device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, const int32_t *__restrict__ a_add,
                                          const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
                                          const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0,
                                          int unit0, int width) {
@@ -671,49 +719,45 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         }
     }
 
-    // packed operand fragments of one k-pair: pf[0..3] the four token sub-tiles, pf[4..] the channel sub-tiles
-    auto frag_read = [&](v4i (&f)[8], int slot, int j) {
-        const uint8_t *sb = lds + slot * kStageB + rd_j[j];
-#pragma unroll
-        for (int b = 0; b < 4; b++) f[b] = *reinterpret_cast<const v4i *>(sb + rd_t + b * 32 * kRowB);
-#pragma unroll
-        for (int a = 0; a < NA; a++) f[4 + a] = *reinterpret_cast<const v4i *>(sb + rd_c + a * 32 * kRowB);
-    };
-    // split the fragments in registers and run the two k-steps they hold
-    auto multiply = [&](const v4i (&f)[8]) {
-        v4i te[4], to[4];
-#pragma unroll
-        for (int b = 0; b < 4; b++) split16(f[b], te[b], to[b]);
-#pragma unroll
-        for (int a = 0; a < NA; a++) {
-            v4i ce, co;
-            split16(f[4 + a], ce, co);
-#pragma unroll
-            for (int b = 0; b < 4; b++) acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te[b], acc[a][b], 0, 0, 0);
-#pragma unroll
-            for (int b = 0; b < 4; b++) acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to[b], acc[a][b], 0, 0, 0);
-        }
-    };
-
-    // On entry pf[0..3] hold the token fragments of (stage pp.it, k-pair 0), read by the previous tile's last
-    // stage (token rows do not depend on the tile); the channel rows do, so their fragments are read here.
-    {
-        const uint8_t *sb = lds + (pp.it % kStages) * kStageB + rd_j[0];
-#pragma unroll
-        for (int a = 0; a < NA; a++) pf[4 + a] = *reinterpret_cast<const v4i *>(sb + rd_c + a * 32 * kRowB);
-    }
-    for (int kt = 0; kt < nk; kt++) {
-        const int slot = pp.it % kStages;
-        frag_read(pg, slot, 1);                     // k-pair 1 of this stage
-        multiply(pf);
-        // stage pp.it + 1 must have landed everywhere before its first fragments are read below; the slot of
-        // stage pp.it - 1 is free for the loads of stage pp.it + kStages - 1 once everyone is past this barrier
+    // ---- main loop: while one k-pair is multiplied the next is read from LDS and split ------------------------------
+    // stage s = pp.it + kt; k-pair j of a stage is the 16-byte chunk 2 j + lg of each 64-byte stage row
+    auto tok_base = [&](int slot, int j) { return lds + slot * kStageB + rd_j[j] + rd_t; };
+    auto chn_base = [&](int slot, int j) { return lds + slot * kStageB + rd_j[j] + rd_c; };
+    // stage s + 1 must have landed everywhere before its fragments are read; the slot of stage s - 1 is free for
+    // the loads of stage s + kStages - 1 once everyone is past this barrier
+    auto sync = [&]() {
         if (pp.store_syncs > 0) { wait_stage(pp.store_extra); pp.store_syncs--; } else { wait_stage(0); }
         plain_barrier();
         loader_issue(ldr, ld, lds, lane);
-        frag_read(pf, (pp.it + 1) % kStages, 0);    // k-pair 0 of the next stage (maybe the next tile's)
-        multiply(pg);
-        pp.it++;
+    };
+    auto no_sync = []() {};
+    if constexpr (NA == 0) {
+        for (int kt = 0; kt < nk; kt++) { sync(); pp.it++; }
+    } else {
+        Frags u0, u1;
+        {   // prologue: the first k-pair of the tile's first stage (landed: the previous synchronisation saw to it)
+            const int slot = pp.it % kStages;
+            const uint8_t *t0 = tok_base(slot, 0), *c0 = chn_base(slot, 0);
+#pragma unroll
+            for (int f = 0; f < 4 + NA; f++) {
+                const v4i raw = *reinterpret_cast<const v4i *>(f < 4 ? t0 + f * 32 * kRowB : c0 + (f - 4) * 32 * kRowB);
+                v4i ev, od;
+                split16(raw, ev, od);
+                if (f < 4) { u0.te[f] = ev; u0.to[f] = od; } else { u0.ce[f - 4] = ev; u0.co[f - 4] = od; }
+            }
+        }
+        for (int kt = 0; kt < nk - 1; kt++) {
+            const int slot = pp.it % kStages, next = (pp.it + 1) % kStages;
+            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync);
+            k_pair<NA, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync);
+            pp.it++;
+        }
+        {   // last stage of the tile: nothing of the next tile is read here (its channel rows sit elsewhere)
+            const int slot = pp.it % kStages;
+            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync);
+            k_pair<NA, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync);
+            pp.it++;
+        }
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
@@ -883,7 +927,7 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     ldr.issued = 0;
     loader_offsets(ldr, ld, lane);
 
-    // ---- pipeline prologue: stages 0 .. kStages - 2 in flight, fragments of (stage 0, k-pair 0) in registers
+    // ---- pipeline prologue: stages 0 .. kStages - 2 in flight, stage 0 landed
 #pragma unroll
     for (int s = 0; s < kStages - 1; s++) loader_issue(ldr, ld, lds, lane);
     wait_vmcnt_imm<kLoads * (kStages - 2)>();
@@ -893,24 +937,12 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     pp.store_extra = OUT != OUT_INT32 ? 4 : 0;   // the first tile's four vector loads
     pp.store_syncs = OUT != OUT_INT32 ? kStages - 2 : 0;
     pp.vec_par = 0;
-    v4i pf[8], pg[8];
-    {
-        const int li = lane & 31, lg = lane >> 5;
-        const uint8_t *sb = lds + ((0 + lg) ^ ((li >> 2) & 3)) * 16;
-#pragma unroll
-        for (int b = 0; b < 4; b++) pf[b] = *reinterpret_cast<const v4i *>(sb + ((wave >> 1) * 128 + li + b * 32) * kRowB);
-#pragma unroll
-        for (int a = 0; a < 4; a++) pf[4 + a] = pf[0];
-#pragma unroll
-        for (int i = 0; i < 8; i++) pg[i] = pf[0];
-    }
-
     while (cc.valid) {
         const int h0 = (cc.width + 1) >> 1;
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
 #define QUEST_BIG_TILE(NA) \
-    big_tile<OUT, NA>(lds, ld, ldr, pp, pf, pg, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
+    big_tile<OUT, NA>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
         switch (na) {
             case 4: QUEST_BIG_TILE(4); break;
             case 3: QUEST_BIG_TILE(3); break;
