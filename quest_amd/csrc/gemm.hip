@@ -601,6 +601,13 @@ __device__ __forceinline__ void wait_stage(int extra) {
     }
 }
 
+// lane number from the execution mask (volatile: never merged with an earlier copy)
+__device__ __forceinline__ int fresh_lane_id() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
 struct Pipe {            // state that lives across tiles
     int it;              // stages multiplied so far (slot = it % kStages)
     int store_extra;     // epilogue stores that may still be in flight ...
@@ -674,7 +681,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     constexpr int NAX = NA > 0 ? NA : 1;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps everything derived from it in scalar registers
     const int wt = wave >> 1;
     const int li = lane & 31;
     const int lg = lane >> 5;
@@ -761,10 +768,15 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
-    // Accumulator register r of lane (li, lg) is channel 8 (r/4) + 4 lg + r%4 of token li: a lane owns
+    // Accumulator register r of lane_e (li_e, lg_e) is channel 8 (r/4) + 4 lg_e + r%4 of token li_e: a lane_e owns
     // 4 consecutive channels.  Storing those directly would write 8- or 16-byte pieces of each output
     // row.  Each wave instead passes 32 tokens x 64 channels (32 for int32) at a time through its own LDS
-    // strip and writes 128-byte runs of each row, 16 bytes per lane.
+    // strip and writes 128-byte runs of each row, 16 bytes per lane_e.
+    // The lane's coordinates are derived afresh here: values kept alive across the main loop would be spilled to
+    // scratch there, and a scratch reload waits on the vector-memory counter, i.e. on every store issued before it.
+    const int lane_e = fresh_lane_id();
+    const int li_e = lane_e & 31;
+    const int lg_e = lane_e >> 5;
     constexpr int kEs = OUT == OUT_INT32 ? 4 : 2;                  // bytes per output element
     constexpr int kApp = OUT == OUT_INT32 ? 1 : 2;                 // channel sub-tiles per pass
     const bool fast = (N % (16 / kEs)) == 0;
@@ -773,11 +785,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         uint8_t *ebuf = lds + kEpiOff + wave * kEpiWaveB;
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            int t_add = 0;                                         // of the token whose values this lane converts
+            int t_add = 0;                                         // of the token whose values this lane_e converts
             float t_half_mul = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                t_add = w_add[wt * 128 + b * 32 + li];
-                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li]));
+                t_add = w_add[wt * 128 + b * 32 + li_e];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
             }
 #pragma unroll
             for (int a0 = 0; a0 < NA; a0 += kApp) {
@@ -790,15 +802,15 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                     if (a >= NA) continue;
 #pragma unroll
                     for (int rg = 0; rg < 4; rg++) {
-                        const int col = aa * 32 + rg * 8 + lg * 4;            // channel inside this pass
+                        const int col = aa * 32 + rg * 8 + lg_e * 4;            // channel inside this pass
                         int c[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++) c[e] = acc[a < NAX ? a : 0][b][rg * 4 + e] >> 8;
-                        uint8_t *dst = ebuf + li * kEpiStride + col * kEs;
+                        uint8_t *dst = ebuf + li_e * kEpiStride + col * kEs;
                         if constexpr (OUT == OUT_INT32) {
                             *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
                         } else {
-                            const int cl = (unit0 + a) * 32 + rg * 8 + lg * 4;   // channel inside the tile
+                            const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;   // channel inside the tile
                             const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
                             const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
                             const int adds[4] = {va.x, va.y, va.z, va.w};
@@ -818,7 +830,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                 const int pieces = cnt * 2 * kEs;
 #pragma unroll
                 for (int i = 0; i < kApp * kEs; i++) {
-                    const int idx = i * 64 + lane;
+                    const int idx = i * 64 + lane_e;
                     const int row = idx / pieces;
                     const int ck = idx - row * pieces;
                     const int tok = tok0 + wt * 128 + b * 32 + row;
@@ -834,19 +846,19 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         // generic path (N not a multiple of 8 / 4): element-wise stores straight from the accumulators
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            const int tok = tok0 + wt * 128 + b * 32 + li;
+            const int tok = tok0 + wt * 128 + b * 32 + li_e;
             if (tok >= M) continue;
             int t_add = 0;
             float t_half_mul = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                t_add = w_add[wt * 128 + b * 32 + li];
-                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li]));
+                t_add = w_add[wt * 128 + b * 32 + li_e];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
             }
 #pragma unroll
             for (int a = 0; a < NA; a++) {
 #pragma unroll
                 for (int rg = 0; rg < 4; rg++) {
-                    const int cl = (unit0 + a) * 32 + rg * 8 + lg * 4;
+                    const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int ch = ch0 + cl + e;
