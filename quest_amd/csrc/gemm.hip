@@ -506,13 +506,10 @@ constexpr int kTileB = kRows * kRowB;         // 16 KiB
 constexpr int kStageB = 2 * kTileB;           // token tile + channel tile
 constexpr int kStages = 4;
 constexpr int kLoads = 8;                     // buffer loads per wave per stage
-constexpr int kEpiStride = 136;               // bytes per token row of the epilogue transposition buffer
-constexpr int kEpiWaveB = 32 * kEpiStride;
-constexpr int kEpiOff = kStages * kStageB;
-constexpr int kVecOff = kEpiOff + 4 * kEpiWaveB;
+constexpr int kVecOff = kStages * kStageB;
 constexpr int kVecParB = 2 * (kRows * 4 + kRows * 2);   // b_add, b_mul per channel and a_add, a_mul per token of one tile
 constexpr int kVecB = 2 * kVecParB;                       // two tiles in flight
-constexpr int kLdsB = kVecOff + kVecB;        // ~148 KiB of the CU's 160 KiB
+constexpr int kLdsB = kVecOff + kVecB;        // 134 KiB of the CU's 160 KiB
 
 // s_barrier alone: waves order their own LDS traffic with s_waitcnt, and a release / acquire fence here would
 // make the compiler drain every direct-to-LDS load still in flight (vmcnt(0)), which is the pipeline
@@ -768,76 +765,83 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
-    // Accumulator register r of lane_e (li_e, lg_e) is channel 8 (r/4) + 4 lg_e + r%4 of token li_e: a lane_e owns
-    // 4 consecutive channels.  Storing those directly would write 8- or 16-byte pieces of each output
-    // row.  Each wave instead passes 32 tokens x 64 channels (32 for int32) at a time through its own LDS
-    // strip and writes 128-byte runs of each row, 16 bytes per lane_e.
+    // Accumulator register r of lane (li, lg) is channel 8 (r/4) + 4 lg + r%4 of token li: a lane owns 4 consecutive
+    // channels of each group of 8.  For 16-bit outputs the two half-waves trade register groups (v_permlane32_swap:
+    // the lower half keeps group g and receives the upper half's part of it, the upper half does the same with
+    // group g + 1), so that every lane stores 16 bytes = 8 consecutive channels and a half-wave pair covers 32
+    // contiguous bytes of each token row; the four stores of a sub-tile complete its 64-byte row segments in L2.
+    constexpr int kEs = OUT == OUT_INT32 ? 4 : 2;                  // bytes per output element
+    const bool fast = (N % (16 / kEs)) == 0;
+    const bool interior = fast && tok0 + kRows <= M && ch0 + 32 * width <= N;
     // The lane's coordinates are derived afresh here: values kept alive across the main loop would be spilled to
     // scratch there, and a scratch reload waits on the vector-memory counter, i.e. on every store issued before it.
     const int lane_e = fresh_lane_id();
     const int li_e = lane_e & 31;
     const int lg_e = lane_e >> 5;
-    constexpr int kEs = OUT == OUT_INT32 ? 4 : 2;                  // bytes per output element
-    constexpr int kApp = OUT == OUT_INT32 ? 1 : 2;                 // channel sub-tiles per pass
-    const bool fast = (N % (16 / kEs)) == 0;
-    const bool interior = fast && tok0 + kRows <= M && ch0 + 32 * width <= N;
     if (NA > 0 && fast) {
-        uint8_t *ebuf = lds + kEpiOff + wave * kEpiWaveB;
+        int t_add[4];                                              // of the tokens whose values this lane converts
+        float t_half_mul[4];
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            int t_add = 0;                                         // of the token whose values this lane_e converts
-            float t_half_mul = 0.f;
+            t_add[b] = 0;
+            t_half_mul[b] = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                t_add = w_add[wt * 128 + b * 32 + li_e];
-                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
+                t_add[b] = w_add[wt * 128 + b * 32 + li_e];
+                t_half_mul[b] = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
+            }
+        }
+        uint8_t *out_lane = reinterpret_cast<uint8_t *>(out) + ((size_t)(tok0 + wt * 128 + li_e) * N + ch0 + unit0 * 32) * kEs;
+#pragma unroll
+        for (int a = 0; a < NA; a++) {
+            int adds[16];
+            float muls[16];
+            if constexpr (OUT != OUT_INT32) {
+#pragma unroll
+                for (int rg = 0; rg < 4; rg++) {
+                    const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;      // channel inside the tile
+                    const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
+                    const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
+                    adds[rg * 4 + 0] = va.x; adds[rg * 4 + 1] = va.y; adds[rg * 4 + 2] = va.z; adds[rg * 4 + 3] = va.w;
+                    muls[rg * 4 + 0] = lo_f32<DT>(vm.x); muls[rg * 4 + 1] = hi_f32<DT>(vm.x);
+                    muls[rg * 4 + 2] = lo_f32<DT>(vm.y); muls[rg * 4 + 3] = hi_f32<DT>(vm.y);
+                }
             }
 #pragma unroll
-            for (int a0 = 0; a0 < NA; a0 += kApp) {
-                constexpr int dummy = 0;
-                (void)dummy;
-                const int cnt = (NA - a0) < kApp ? (NA - a0) : kApp;
-#pragma unroll
-                for (int aa = 0; aa < kApp; aa++) {
-                    const int a = a0 + aa;
-                    if (a >= NA) continue;
+            for (int b = 0; b < 4; b++) {
+                const bool tok_ok = tok0 + wt * 128 + b * 32 + li_e < M;
+                uint8_t *dst = out_lane + ((size_t)b * 32 * N + a * 32) * kEs;
+                if constexpr (OUT == OUT_INT32) {
 #pragma unroll
                     for (int rg = 0; rg < 4; rg++) {
-                        const int col = aa * 32 + rg * 8 + lg_e * 4;            // channel inside this pass
-                        int c[4];
-#pragma unroll
-                        for (int e = 0; e < 4; e++) c[e] = acc[a < NAX ? a : 0][b][rg * 4 + e] >> 8;
-                        uint8_t *dst = ebuf + li_e * kEpiStride + col * kEs;
-                        if constexpr (OUT == OUT_INT32) {
-                            *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
-                        } else {
-                            const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;   // channel inside the tile
-                            const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
-                            const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
-                            const int adds[4] = {va.x, va.y, va.z, va.w};
-                            const float muls[4] = {lo_f32<DT>(vm.x), hi_f32<DT>(vm.x), lo_f32<DT>(vm.y), hi_f32<DT>(vm.y)};
-                            uint32_t h[4];
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                const float lhs = (float)(c[e] * 2 + t_add + adds[e]);
-                                const float rhs = __fmul_rn(t_half_mul, muls[e]);
-                                h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
-                            }
-                            *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-                        }
+                        const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;
+                        if (tok_ok && ch0 + cl < N)
+                            *reinterpret_cast<int4 *>(dst + (rg * 8 + lg_e * 4) * 4) =
+                                make_int4(acc[a][b][rg * 4] >> 8, acc[a][b][rg * 4 + 1] >> 8, acc[a][b][rg * 4 + 2] >> 8,
+                                          acc[a][b][rg * 4 + 3] >> 8);
                     }
-                }
-                // rows back out: 32 rows x (cnt * 32 channels) in 16-byte pieces
-                const int pieces = cnt * 2 * kEs;
+                } else {
+                    uint32_t x[4][2];
 #pragma unroll
-                for (int i = 0; i < kApp * kEs; i++) {
-                    const int idx = i * 64 + lane_e;
-                    const int row = idx / pieces;
-                    const int ck = idx - row * pieces;
-                    const int tok = tok0 + wt * 128 + b * 32 + row;
-                    const int ch = ch0 + (unit0 + a0) * 32 + ck * (16 / kEs);
-                    if (row < 32 && tok < M && ch < N) {
-                        const uint4 v = *reinterpret_cast<const uint4 *>(ebuf + row * kEpiStride + ck * 16);
-                        *reinterpret_cast<uint4 *>(reinterpret_cast<uint8_t *>(out) + ((size_t)tok * N + ch) * kEs) = v;
+                    for (int rg = 0; rg < 4; rg++) {
+                        uint32_t h[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int c = acc[a][b][rg * 4 + e] >> 8;
+                            const float lhs = (float)(c * 2 + t_add[b] + adds[rg * 4 + e]);
+                            const float rhs = __fmul_rn(t_half_mul[b], muls[rg * 4 + e]);
+                            h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
+                        }
+                        x[rg][0] = h[0] | (h[1] << 16);
+                        x[rg][1] = h[2] | (h[3] << 16);
+                    }
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++) {
+                        // lower half-wave: group 2 pr complete; upper half-wave: group 2 pr + 1 complete
+                        const auto s0 = __builtin_amdgcn_permlane32_swap(x[2 * pr][0], x[2 * pr + 1][0], false, false);
+                        const auto s1 = __builtin_amdgcn_permlane32_swap(x[2 * pr][1], x[2 * pr + 1][1], false, false);
+                        const int cl = (unit0 + a) * 32 + (2 * pr + lg_e) * 8;
+                        if (tok_ok && ch0 + cl < N)
+                            *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
                     }
                 }
             }
