@@ -559,26 +559,33 @@ __device__ __forceinline__ void loader_offsets(Loader &l, const Cursor &ld, int 
     l.off_c = (uint32_t)(ld.ch0 + row) * (uint32_t)l.kbytes + chunk * 16;
 }
 
-// Issue the load cursor's stage into the next LDS slot, then advance the cursor (into the next tile
-// when this one is done; when nothing is left the last stage is fetched again, which keeps the
-// count of outstanding loads uniform).  Rows past the end of a matrix read as zeros.
-__device__ __forceinline__ void loader_issue(Loader &l, Cursor &ld, uint8_t *lds, int lane) {
+// The load cursor's stage goes into the next LDS slot as eight instructions per wave (loader_one, j = 0..7: four of
+// 16 token rows, four of 16 channel rows), issued a few MFMAs apart because each takes the CU's address path about
+// half an MFMA; loader_end then advances the cursor (into the next tile when this one is done; when nothing is
+// left the last stage is fetched again, which keeps the count of outstanding loads uniform).
+// Rows past the end of a matrix read as zeros.
+__device__ __forceinline__ void loader_one(const Loader &l, const Cursor &ld, uint8_t *lds, int j) {
     uint8_t *sb = lds + (l.issued % kStages) * kStageB + l.wave * 64 * kRowB;
     const int kb = ld.kt * kRowB;
     const int step = 16 * l.kbytes;
-#pragma unroll
-    for (int j = 0; j < 4; j++)
+    if (j < 4)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(l.act, (__attribute__((address_space(3))) void *)(sb + j * 16 * kRowB), 16,
                                                  l.off_t, kb + j * step, 0, 0);
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.wgt, (__attribute__((address_space(3))) void *)(sb + kTileB + j * 16 * kRowB),
-                                                 16, l.off_c, kb + j * step, 0, 0);
+    else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.wgt, (__attribute__((address_space(3))) void *)(sb + kTileB + (j - 4) * 16 * kRowB),
+                                                 16, l.off_c, kb + (j - 4) * step, 0, 0);
+}
+__device__ __forceinline__ void loader_end(Loader &l, Cursor &ld, int lane) {
     l.issued++;
     if (++ld.kt == l.nk) {
         cursor_next_tile(ld);
         if (ld.valid) loader_offsets(l, ld, lane); else ld.kt = l.nk - 1;
     }
+}
+__device__ __forceinline__ void loader_issue(Loader &l, Cursor &ld, uint8_t *lds, int lane) {
+#pragma unroll
+    for (int j = 0; j < kLoads; j++) loader_one(l, ld, lds, j);
+    loader_end(l, ld, lane);
 }
 
 template <int N>
@@ -630,12 +637,12 @@ struct Frags {
 // between them and the order pinned (a lone wave per SIMD issues in order: VALU work, LDS reads and the stage
 // synchronisation only overlap the matrix pipe if they sit between MFMAs, which are 32 cycles apart):
 //   * the MFMAs of this k-pair, operands in `cur`;
-//   * `sync` runs after slot kSyncSlot (-1: none);
+//   * `sync` runs after slot kSyncSlot (-1: none) and the stage's loads, dma(0..kLoads), follow one per few slots;
 //   * NEXT: the packed fragments of the next k-pair are read from LDS in the slots after that, up to 3/8 of the
 //     way, and split into `nxt` (3 VALU ops per dword) over the second half of the slots.
-template <int NA, bool NEXT, int kSyncSlot, typename Sync>
+template <int NA, bool NEXT, int kSyncSlot, typename Sync, typename Dma>
 __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Frags &cur, Frags &nxt, const uint8_t *rd_tok,
-                                       const uint8_t *rd_chn, Sync &&sync) {
+                                       const uint8_t *rd_chn, Sync &&sync, Dma &&dma) {
     constexpr int S = 8 * NA;                 // slots
     constexpr int F = 4 + NA;                 // fragments per k-pair
     constexpr int V = F * 4;                  // dwords to split
@@ -649,6 +656,13 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
         acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(odd ? cur.co[a] : cur.ce[a], odd ? cur.to[b] : cur.te[b], acc[a][b],
                                                           0, 0, 0);
         if (i == kSyncSlot) sync();
+        if constexpr (kSyncSlot >= 0) {
+            // the stage's kLoads direct-to-LDS loads and the cursor step (item kLoads), spread over the remaining slots
+            if (i > kSyncSlot) {
+#pragma unroll
+                for (int j = (i - R0) * (kLoads + 1) / (S - R0); j < (i - R0 + 1) * (kLoads + 1) / (S - R0); j++) dma(j);
+            }
+        }
         if constexpr (NEXT) {
             if (i >= R0 && i < R1) {
 #pragma unroll
@@ -732,11 +746,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     auto sync = [&]() {
         if (pp.store_syncs > 0) { wait_stage(pp.store_extra); pp.store_syncs--; } else { wait_stage(0); }
         plain_barrier();
-        loader_issue(ldr, ld, lds, lane);
     };
+    auto dma = [&](int j) { if (j < kLoads) loader_one(ldr, ld, lds, j); else loader_end(ldr, ld, lane); };
     auto no_sync = []() {};
     if constexpr (NA == 0) {
-        for (int kt = 0; kt < nk; kt++) { sync(); pp.it++; }
+        for (int kt = 0; kt < nk; kt++) { sync(); loader_issue(ldr, ld, lds, lane); pp.it++; }
     } else {
         Frags u0, u1;
         {   // prologue: the first k-pair of the tile's first stage (landed: the previous synchronisation saw to it)
@@ -752,14 +766,14 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         }
         for (int kt = 0; kt < nk - 1; kt++) {
             const int slot = pp.it % kStages, next = (pp.it + 1) % kStages;
-            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync);
-            k_pair<NA, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync);
+            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
+            k_pair<NA, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync, dma);
             pp.it++;
         }
         {   // last stage of the tile: nothing of the next tile is read here (its channel rows sit elsewhere)
             const int slot = pp.it % kStages;
-            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync);
-            k_pair<NA, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync);
+            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
+            k_pair<NA, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync, dma);
             pp.it++;
         }
     }
