@@ -62,6 +62,14 @@ __device__ __forceinline__ uint32_t pack2_rne(float lo, float hi) {
     }
 }
 
+// Two fp32 products rounded to the dtype and packed.  The empty asm pins both as fp32 registers (see from_f32), then
+// one two-element conversion rounds each to nearest even.
+template <int DT>
+__device__ __forceinline__ uint32_t pack2_rounded_products(float lo, float hi) {
+    asm volatile("" : "+v"(lo), "+v"(hi));
+    return pack2_rne<DT>(lo, hi);
+}
+
 // ---- cross-lane moves -----------------------------------------------------------------------
 // value of lane (lane ^ M); M = 1, 2, 8 are single DPP moves, 4 and 16 LDS-crossbar swizzles.
 template <int M>

@@ -837,16 +837,16 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                     uint32_t x[4][2];
 #pragma unroll
                     for (int rg = 0; rg < 4; rg++) {
-                        uint32_t h[4];
+                        float v[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            const int c = acc[a][b][rg * 4 + e] >> 8;
-                            const float lhs = (float)(c * 2 + t_add[b] + adds[rg * 4 + e]);
+                            // the accumulator is 256 C exactly, so 2 C is one arithmetic shift
+                            const float lhs = (float)((acc[a][b][rg * 4 + e] >> 7) + t_add[b] + adds[rg * 4 + e]);
                             const float rhs = __fmul_rn(t_half_mul[b], muls[rg * 4 + e]);
-                            h[e] = from_f32<DT>(__fmul_rn(lhs, rhs));
+                            v[e] = __fmul_rn(lhs, rhs);
                         }
-                        x[rg][0] = h[0] | (h[1] << 16);
-                        x[rg][1] = h[2] | (h[3] << 16);
+                        x[rg][0] = pack2_rounded_products<DT>(v[0], v[1]);
+                        x[rg][1] = pack2_rounded_products<DT>(v[2], v[3]);
                     }
 #pragma unroll
                     for (int pr = 0; pr < 2; pr++) {
