@@ -33,10 +33,10 @@ HBM_PEAK_GBS = 8000.0
 INT8_MFMA_PEAK_TOPS = 5000.0
 
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
-# scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.99979, WRITE_SIZE x 1.0);
+# scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.99980, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
-TRAFFIC_GEMM_BYTES = int((128273.8 * 1.99979 + 109677.0) * 1024)        # M=4096 K=4096 N=11008 fp16
-TRAFFIC_QUANTIZE_BYTES = int((32814.8 * 1.99979 + 16512.9) * 1024)      # bf16 [8192, 4096]
+TRAFFIC_GEMM_BYTES = 358800835          # M=4096 K=4096 N=11008 fp16: (118931.1 x 1.99980 + 112553.2) KiB
+TRAFFIC_QUANTIZE_BYTES = 84105907       # bf16 [8192, 4096]: (32814.2 x 1.99980 + 16512.9) KiB
 
 
 def event_pairs(n):
@@ -113,17 +113,26 @@ def bench_linear(quest, _lib, steps, warmup, dev):
     quant_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
     gemm_in_step_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
 
-    # the GEMM alone, bare C-ABI launches on the codes the last step left
+    # the GEMM alone, bare C-ABI launches: on uniform random activation codes (the stated GEMM workload; the
+    # matrix cores draw the most power on them) and on the codes the last step left (Gaussian activations)
     lib = _lib.load()
     st = _lib.stream_of(out)
-    args = (_lib.ptr(out), _lib.ptr(a_packed), _lib.ptr(w_packed), _lib.ptr(a_row_sum), _lib.ptr(w_add),
-            _lib.ptr(a_scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype], st)       # sizes in the ABI's order: M, K, N
+    u_codes = torch.randint(-8, 8, (m, k), generator=g, dtype=torch.int8)
+    u_packed = ((u_codes[:, 1::2] << 4) | (u_codes[:, ::2] & 0xF)).view(torch.uint8).to(dev)
+    u_row_sum = u_codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32).to(dev)
+    u_scale = (torch.rand(m, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
 
-    def gemm(_):
-        if lib.quest_fused_matmul_dequantize_int4_int4t(*args) != 0:
-            raise RuntimeError('GEMM launch failed')
+    def gemm_launcher(codes, row_sum, scale):
+        args = (_lib.ptr(out), _lib.ptr(codes), _lib.ptr(w_packed), _lib.ptr(row_sum), _lib.ptr(w_add),
+                _lib.ptr(scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype], st)     # sizes in the ABI's order: M, K, N
 
-    gemm_ms = launches_ms(gemm, max(steps, 20))
+        def gemm(_):
+            if lib.quest_fused_matmul_dequantize_int4_int4t(*args) != 0:
+                raise RuntimeError('GEMM launch failed')
+        return gemm
+
+    gemm_quantized_ms = launches_ms(gemm_launcher(a_packed, a_row_sum, a_scale), max(steps, 100))
+    gemm_ms = launches_ms(gemm_launcher(u_packed, u_row_sum, u_scale), max(steps, 100))
     ops = 2.0 * m * n * k
     return {
         'shape': {'M': m, 'K': k, 'N': n},
@@ -132,6 +141,7 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         'gemm_ms': gemm_ms,
         'gemm_tops': ops / (gemm_ms * 1e-3) / 1e12,
         'gemm_in_step_ms': gemm_in_step_ms,
+        'gemm_quantized_acts_ms': gemm_quantized_ms,
         'quant_ms': quant_ms,
     }
 
@@ -254,7 +264,7 @@ def calibration_stream(dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     args = ap.parse_args()
@@ -270,7 +280,7 @@ def main():
     torch.cuda.set_device(dev)
 
     lin = bench_linear(quest, _lib, args.steps, args.warmup, dev)
-    rq = bench_quantize(_lib, max(args.steps, 60), args.warmup, dev)
+    rq = bench_quantize(_lib, max(args.steps, 100), args.warmup, dev)
     dec = bench_decode(_lib, dev)
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
@@ -278,7 +288,8 @@ def main():
     roofline = {'bound': 'mfma', 'achieved': lin['gemm_tops'], 'peak': INT8_MFMA_PEAK_TOPS, 'unit': 'TOP/s',
                 'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES,
                 'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
-                'algorithmic_ops': 2.0 * 4096 * 4096 * 11008}
+                'algorithmic_ops': 2.0 * 4096 * 4096 * 11008,
+                'workload': 'uniform random INT4 codes on both sides, M=4096 K=4096 N=11008, fp16 out'}
     line = {
         'metric': 'INT4-GEMM TOPS + quantize GB/s at Llama-7B layer shapes, % MI355X roofline',
         'value': lin['tops'], 'unit': 'TOPS', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -288,6 +299,7 @@ def main():
                                'Hadamard-quantize-pack -> packed INT4 GEMM [4096,4096]x[11008,4096]^T -> fp16 [4096,11008]',
                    'M': 4096, 'K': 4096, 'N': 11008},
         'gemm_tops': lin['gemm_tops'], 'gemm_us_in_step': lin['gemm_in_step_ms'] * 1e3,
+        'gemm_tops_on_quantized_activations': 2.0 * 4096 * 4096 * 11008 / (lin['gemm_quantized_acts_ms'] * 1e-3) / 1e12,
         'quantize_us_in_step': lin['quant_ms'] * 1e3,
         'quantize_GBs': rq['achieved'],
         'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'cpu_baseline': cpu,
