@@ -13,6 +13,7 @@ are converted).  The JSON line also carries
   roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
                      outlier channels) against the HBM peak,
   decode             the layer at M in {1, 8, 16}: the weight-streaming GEMM alone and with the activation kernel,
+  forward            the 12-layer Llama of the reference's end-to-end benchmark, dense vs W4A4 vs no-op linears,
   cpu_baseline       the CPU oracle (PyTorch restatement of the reference's `backend='pytorch'`
                      path) on the reference's CPU-runnable case, timed on this host's cores.
 """
@@ -215,6 +216,33 @@ def bench_decode(_lib, dev):
     return out
 
 
+def bench_forward(dev):
+    """The whole-model row: 12-layer d=1024 Llama, ids (32, 512), bf16, every transformer projection W4A4 with the
+    Hadamard on.  Times per forward for the dense model, the INT4 model and the no-op model (everything but the
+    linears); the linear-only fraction prices (int4 - noop) against the INT8 matrix peak."""
+    from quest_amd import llama
+    out = {}
+    cfg = llama.LlamaConfig()
+    batch, seq = 32, cfg.sequence_length
+    for mode in ('bf16', 'int4', 'noop'):
+        torch.manual_seed(0)
+        model = llama.Llama(cfg).to(torch.bfloat16).to(dev).eval()
+        llama.quantize_model(model, mode, use_hadamard=True, fuse_gate_up=True)
+        r = llama.bench_forward(model, batch, seq)
+        out[mode] = {'eager_ms': r['eager_s'] * 1e3, 'graph_ms': r['graph_s'] * 1e3, 'best_ms': r['best_s'] * 1e3,
+                     'graph_matches_eager': r['graph_matches_eager']}
+        del model
+        torch.cuda.empty_cache()
+    ops = cfg.linear_ops_per_token() * batch * seq
+    lin_ms = out['int4']['best_ms'] - out['noop']['best_ms']
+    return {'model': '12 layers, d=1024, 16 heads, SwiGLU 2816, vocab 32000, random init', 'tokens': batch * seq,
+            'modes': out, 'int4_tokens_per_s': batch * seq / (out['int4']['best_ms'] * 1e-3),
+            'speedup_over_bf16': out['bf16']['best_ms'] / out['int4']['best_ms'],
+            'linear_int_ops': ops, 'linear_ms': lin_ms,
+            'linear_frac_of_int8_peak': ops / (lin_ms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS,
+            'wiring': 'QKV fused (as the reference); gate and up share one quantisation and one GEMM'}
+
+
 def bench_cpu_baseline():
     """The CPU oracle on the reference's CPU-runnable case: fp16 [512,1024] x [1024,1024]^T, Hadamard
     as F.linear, scale, quantise, integer GEMM through fp64 as the reference's own check does, and
@@ -267,6 +295,7 @@ def main():
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-forward', action='store_true', help='skip the whole-model row')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build runs on one GPU; --gpus above 1 is not supported '
@@ -282,6 +311,7 @@ def main():
     lin = bench_linear(quest, _lib, args.steps, args.warmup, dev)
     rq = bench_quantize(_lib, max(args.steps, 100), args.warmup, dev)
     dec = bench_decode(_lib, dev)
+    fwd = None if args.no_forward else bench_forward(dev)
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
 
@@ -302,7 +332,7 @@ def main():
         'gemm_tops_on_quantized_activations': 2.0 * 4096 * 4096 * 11008 / (lin['gemm_quantized_acts_ms'] * 1e-3) / 1e12,
         'quantize_us_in_step': lin['quant_ms'] * 1e3,
         'quantize_GBs': rq['achieved'],
-        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'cpu_baseline': cpu,
+        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'forward': fwd, 'cpu_baseline': cpu,
     }
     print(json.dumps(line))
 

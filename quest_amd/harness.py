@@ -157,6 +157,21 @@ class Linear4bit(nn.Module):
         self.register_buffer('w_meta_e', None)
         return self
 
+    @classmethod
+    def empty(cls, in_features: int, out_features: int, bias: bool = False, device=None, dtype=None,
+              use_hadamard: bool = False) -> 'Linear4bit':
+        """A layer of the given shape with unset buffers, to be filled by `load_state_dict` from a packed checkpoint."""
+        self = cls.__new__(cls)
+        nn.Module.__init__(self)
+        self.use_hadamard, self.use_noop = use_hadamard, False
+        self.bias = nn.Parameter(torch.zeros(out_features, dtype=dtype, device=device)) if bias else None
+        self.weight = torch.empty(out_features, in_features, dtype=dtype, device=torch.device('meta'))
+        self.register_buffer('w_int_packed', torch.zeros(out_features, in_features // 2, dtype=torch.uint8, device=device))
+        self.register_buffer('w_scale', torch.zeros(out_features, 1, dtype=dtype, device=device))
+        self.register_buffer('w_add', torch.zeros(out_features, 1, dtype=torch.int32, device=device))
+        self.register_buffer('w_meta_e', None)
+        return self
+
     def forward(self, x) -> torch.Tensor:
         if not self.use_noop:
             a = x.contiguous().flatten(end_dim=-2)

@@ -1,0 +1,246 @@
+"""The Llama-style decoder the reference benchmarks end to end, with every transformer projection as a W4A4
+linear on the HIP kernels.
+
+Mirrors the model the reference builds for gemm-quest/benchmarks/bench_e2e.py (src/models/llama.py:17-62 RoPE,
+65-77 RMSNorm, 79-118 SwiGLU MLP, 121-177 attention and block, 180-247 model; src/models/base.py:32-60 fused
+QKV `c_attn` + `c_proj`; init src/models/base.py:98-104 and llama.py:213-217) and the layer swap of
+bench_e2e.py:73-99: only the linears under `transformer` are replaced, `lm_head` stays a dense bf16 matmul.
+Module names follow the reference (`transformer.h.<i>.attn.c_attn`, `mlp.w1`, ...), so a state dict of the
+reference's model loads by name.
+
+Modes (bench_e2e.py:84-95): 'bf16' dense torch linears, 'int4' packed INT4 weights and the W4A4 kernels,
+'noop' the same modules returning zeros (everything but the linears).  Two things differ from the reference's
+'int4' wiring, both switchable: gate and up projections (`w1`, `w2`) read the same tensor, so it is quantised
+once and multiplied by the concatenated weights in one GEMM (`fuse_gate_up`); the reference launches them
+separately (llama.py:89-106, 117-118).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+from . import harness
+
+
+@dataclass
+class LlamaConfig:
+    """Defaults: the 12-layer, d=1024 model of the end-to-end benchmark row."""
+    n_layer: int = 12
+    n_embd: int = 1024
+    n_head: int = 16
+    multiple_of: int = 256
+    vocab_size: int = 32000
+    sequence_length: int = 512
+    rmsnorm_eps: float = 1e-5
+    init_std: float = 0.02
+    bias: bool = False
+
+    @property
+    def hidden_dim(self) -> int:
+        """llama.py:83-87: 2/3 of 4 d, rounded up to a multiple of `multiple_of` (2816 for d=1024)."""
+        h = int(2 * self.n_embd * 4 / 3)
+        return self.multiple_of * ((h + self.multiple_of - 1) // self.multiple_of)
+
+    def linear_ops_per_token(self) -> int:
+        """Integer operations (2 per multiply-add) of the transformer linears for one token."""
+        d, h = self.n_embd, self.hidden_dim
+        return 2 * self.n_layer * (d * 3 * d + d * d + 2 * d * h + h * d)
+
+
+def precompute_freqs_cis(dim: int, end: int, theta: float = 10000.0) -> torch.Tensor:
+    """llama.py:17-24: (end, dim/2, 2) cos / sin table."""
+    freqs = 1.0 / (theta ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
+    ang = torch.outer(torch.arange(end), freqs).float()
+    return torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1)
+
+
+def apply_rotary_emb(q: torch.Tensor, k: torch.Tensor, freqs_cis: torch.Tensor):
+    """llama.py:43-62: rotate interleaved pairs of q, k (B, T, nh, hs) in fp32, back to the input dtype."""
+    dtype = q.dtype
+    cos = freqs_cis[..., 0].view(1, q.size(1), 1, -1)
+    sin = freqs_cis[..., 1].view(1, q.size(1), 1, -1)
+
+    def rot(x):
+        x = x.float().reshape(*x.shape[:-1], -1, 2)
+        re = x[..., 0] * cos - x[..., 1] * sin
+        im = x[..., 0] * sin + x[..., 1] * cos
+        return torch.stack((re, im), dim=-1).flatten(3).to(dtype)
+
+    return rot(q), rot(k)
+
+
+class RMSNorm(nn.Module):
+    """llama.py:65-77."""
+
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)).type_as(x) * self.weight
+
+
+class LlamaMLP(nn.Module):
+    """llama.py:79-118: c_proj(silu(w1 x) * w2 x)."""
+
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.w1 = nn.Linear(config.n_embd, config.hidden_dim, bias=False)
+        self.w2 = nn.Linear(config.n_embd, config.hidden_dim, bias=False)
+        self.c_proj = nn.Linear(config.hidden_dim, config.n_embd, bias=False)
+        self.w12 = None          # set by quantize_model(..., fuse_gate_up=True): one module for both
+
+    def forward(self, x):
+        if self.w12 is not None:
+            gate_up = self.w12(x)
+            h = gate_up.size(-1) // 2
+            return self.c_proj(F.silu(gate_up[..., :h]) * gate_up[..., h:])
+        return self.c_proj(F.silu(self.w1(x)) * self.w2(x))
+
+
+class LlamaAttention(nn.Module):
+    """base.py:32-60 and llama.py:121-163: fused QKV projection, RoPE on q and k, causal attention, output projection."""
+
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        assert config.n_embd % config.n_head == 0
+        self.c_attn = nn.Linear(config.n_embd, 3 * config.n_embd, bias=config.bias)
+        self.c_proj = nn.Linear(config.n_embd, config.n_embd, bias=config.bias)
+        self.n_head, self.n_embd = config.n_head, config.n_embd
+
+    def forward(self, x, freqs_cis):
+        b, t, c = x.size()
+        q, k, v = self.c_attn(x).split(self.n_embd, dim=2)
+        k = k.view(b, t, self.n_head, c // self.n_head)
+        q = q.view(b, t, self.n_head, c // self.n_head)
+        q, k = apply_rotary_emb(q, k, freqs_cis)
+        q, k = q.transpose(1, 2), k.transpose(1, 2)
+        v = v.view(b, t, self.n_head, c // self.n_head).transpose(1, 2)
+        y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=True)
+        return self.c_proj(y.transpose(1, 2).contiguous().view(b, t, c))
+
+
+class LlamaBlock(nn.Module):
+    """llama.py:166-177."""
+
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.ln_1 = RMSNorm(config.n_embd, eps=config.rmsnorm_eps)
+        self.attn = LlamaAttention(config)
+        self.ln_2 = RMSNorm(config.n_embd, eps=config.rmsnorm_eps)
+        self.mlp = LlamaMLP(config)
+
+    def forward(self, x, freqs_cis):
+        x = x + self.attn(self.ln_1(x), freqs_cis)
+        return x + self.mlp(self.ln_2(x))
+
+
+class Llama(nn.Module):
+    """llama.py:180-247 without tokenizer, dropout (0 at inference) and loss."""
+
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.config = config
+        self.freqs_cis = precompute_freqs_cis(config.n_embd // config.n_head, config.sequence_length)
+        self.transformer = nn.ModuleDict(dict(
+            wte=nn.Embedding(config.vocab_size, config.n_embd),
+            h=nn.ModuleList([LlamaBlock(config) for _ in range(config.n_layer)]),
+            ln_f=RMSNorm(config.n_embd, eps=config.rmsnorm_eps),
+        ))
+        self.lm_head = nn.Linear(config.n_embd, config.vocab_size, bias=False)
+        self.apply(self._init_weights)
+        for name, p in self.named_parameters():
+            if name.endswith('c_proj.weight'):
+                nn.init.normal_(p, mean=0.0, std=config.init_std / math.sqrt(2 * config.n_layer))
+
+    def _init_weights(self, module):
+        if isinstance(module, nn.Linear):
+            nn.init.normal_(module.weight, mean=0.0, std=self.config.init_std)
+            if module.bias is not None:
+                nn.init.zeros_(module.bias)
+        elif isinstance(module, nn.Embedding):
+            nn.init.normal_(module.weight, mean=0.0, std=self.config.init_std)
+
+    def hidden_states(self, idx: torch.Tensor) -> torch.Tensor:
+        """Everything up to and including the final norm: (B, T) ids -> (B, T, d)."""
+        t = idx.size(1)
+        assert t <= self.config.sequence_length
+        x = self.transformer.wte(idx)
+        if self.freqs_cis.device != x.device:          # moved once, outside any graph capture (the table stays fp32)
+            self.freqs_cis = self.freqs_cis.to(x.device)
+        freqs_cis = self.freqs_cis[:t]
+        for block in self.transformer.h:
+            x = block(x, freqs_cis)
+        return self.transformer.ln_f(x)
+
+    def forward(self, idx: torch.Tensor, all_logits: bool = False) -> dict:
+        """Logits of the last position (llama.py:253-262, the reference's inference default) or of all positions."""
+        x = self.hidden_states(idx)
+        logits = self.lm_head(x) if all_logits else self.lm_head(x[:, -1:, :])      # a slice: index lists copy from the host
+        return {'logits': logits}
+
+
+def _pack(linear: nn.Linear, use_hadamard: bool, use_noop: bool) -> harness.Linear4bit:
+    m = harness.Linear4bit.from_weight(linear.weight.data, bias=None if linear.bias is None else linear.bias.data,
+                                       use_hadamard=use_hadamard)
+    m.use_noop = use_noop
+    return m
+
+
+@torch.no_grad()
+def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, fuse_gate_up: bool = True) -> Llama:
+    """bench_e2e.py:77-97 on an existing model: every linear under `transformer` becomes a `Linear4bit` holding the
+    packed INT4 form of that linear's own weight ('int4'), or the same module in no-op mode ('noop'); 'bf16' leaves
+    the dense linears.  The model must already sit on the GPU in bf16 or fp16."""
+    if mode == 'bf16':
+        return model
+    if mode not in ('int4', 'noop'):
+        raise NotImplementedError(mode)
+    noop = mode == 'noop'
+    for block in model.transformer.h:
+        block.attn.c_attn = _pack(block.attn.c_attn, use_hadamard, noop)
+        block.attn.c_proj = _pack(block.attn.c_proj, use_hadamard, noop)
+        mlp = block.mlp
+        if fuse_gate_up:
+            both = nn.Linear(mlp.w1.in_features, 2 * mlp.w1.out_features, bias=False, device=mlp.w1.weight.device,
+                             dtype=mlp.w1.weight.dtype)
+            both.weight.data = torch.cat([mlp.w1.weight.data, mlp.w2.weight.data], dim=0)
+            mlp.w12 = _pack(both, use_hadamard, noop)
+            mlp.w1 = mlp.w2 = None
+        else:
+            mlp.w1 = _pack(mlp.w1, use_hadamard, noop)
+            mlp.w2 = _pack(mlp.w2, use_hadamard, noop)
+        mlp.c_proj = _pack(mlp.c_proj, use_hadamard, noop)
+    return model
+
+
+@torch.inference_mode()
+def bench_forward(model: Llama, batch_size: int, seq_len: int, n_warmup: int = 5, n_iter: int = 10) -> dict:
+    """bench_e2e.py:99-121: seconds per forward, eagerly and as a replayed HIP graph (the smaller is the
+    reference's figure); the graph's logits are checked against the eager ones on fresh ids."""
+    dev = next(model.parameters()).device
+    g = torch.Generator(device='cpu').manual_seed(0)
+    input_ids = torch.randint(0, model.config.vocab_size, (batch_size, seq_len), generator=g).to(dev)
+    f = lambda: model(input_ids)['logits']           # noqa: E731
+    t_eager = harness.do_bench(f, n_iter=n_iter, n_warmup=n_warmup)
+    graph = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(n_warmup):
+            f()
+    torch.cuda.current_stream().wait_stream(s)
+    with torch.cuda.graph(graph):
+        out = f()
+    t_graph = harness.do_bench(graph.replay, n_iter=n_iter, n_warmup=n_warmup)
+    input_ids.copy_(torch.randint(0, model.config.vocab_size, (batch_size, seq_len), generator=g).to(dev))
+    graph.replay()
+    torch.cuda.synchronize()
+    graph_ok = bool(torch.equal(out, f()))
+    return {'eager_s': t_eager, 'graph_s': t_graph, 'best_s': min(t_eager, t_graph), 'graph_matches_eager': graph_ok}
