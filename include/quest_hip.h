@@ -110,6 +110,30 @@ int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t *x_int_pack
                                  int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size,
                                  float had_scale, int dtype, void *stream);
 
+/*
+ * quest_hadamard_quantize_int4 with the producer of the activation in front, so that the normalised tensor is
+ * never written: y = dtype(dtype(f32(x) * rsqrt(mean(x^2) + eps)) * norm_weight) -- the RMSNorm in front of every
+ * attention and MLP block of the reference's model (src/models/llama.py:71-77, applied at llama.py:174-175) --
+ * then Hadamard, scale, codes, row sums of y as above.  x_norm, when not NULL, receives y.  No counterpart in
+ * the reference's quest package, which quantises a tensor the norm has already written.
+ * group_size % 128 == 0, group_size <= 4096, had_scale exactly representable in dtype (181/2048 is);
+ * QUEST_ERR_UNSUPPORTED otherwise (the caller then runs the norm itself and quest_hadamard_quantize_int4).
+ */
+int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *norm_weight, float eps, void *scale,
+                                         uint8_t *x_int_packed, int32_t *x_int_row_sum, void *x_had,
+                                         void *x_norm, int group_size, int batch_size, float had_scale,
+                                         int dtype, void *stream);
+
+/*
+ * The same for the SwiGLU product in front of the MLP's output projection (src/models/llama.py:117-118):
+ * gate_up is (batch_size, 2 * group_size), gate in the first half of each row and up in the second;
+ * y = dtype(dtype(silu(gate)) * up), silu(g) = g / (1 + exp(-g)) in fp32.  x_act, when not NULL, receives y
+ * (batch_size, group_size).  Limits and error behaviour as above.
+ */
+int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *scale, uint8_t *x_int_packed,
+                                          int32_t *x_int_row_sum, void *x_had, void *x_act, int group_size,
+                                          int batch_size, float had_scale, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

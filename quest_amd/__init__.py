@@ -17,6 +17,8 @@ from .api import (  # noqa: F401
     matmul_int4sp_int4t_int32,
     quantize_int4,
     reorder_meta48_int4,
+    rmsnorm_hadamard_quantize_int4,
+    silu_mul_hadamard_quantize_int4,
     uncompress_meta48_int4,
 )
 

@@ -193,3 +193,70 @@ def hadamard_quantize_int4(
                                                        ptr(x_had), k, m, float(hadamard_scale), DTYPE_CODE[x.dtype],
                                                        stream_of(x)), 'hadamard_quantize_int4')
     return scale, x_int_packed, x_int_row_sum
+
+
+def _quant_outputs(m, k, dtype, device, scale, x_int_packed, x_int_row_sum):
+    if scale is None:
+        scale = torch.empty(m, 1, dtype=dtype, device=device)
+    if x_int_packed is None:
+        x_int_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=device)
+    if x_int_row_sum is None:
+        x_int_row_sum = torch.empty(m, 1, dtype=torch.int32, device=device)
+    assert scale.dtype == dtype and x_int_packed.dtype == torch.uint8 and x_int_row_sum.dtype == torch.int32
+    assert scale.is_contiguous() and x_int_packed.is_contiguous() and x_int_row_sum.is_contiguous()
+    assert scale.numel() == m and x_int_row_sum.numel() == m and x_int_packed.shape == (m, k // 2)
+    return scale, x_int_packed, x_int_row_sum
+
+
+def rmsnorm_hadamard_quantize_int4(
+        x: torch.Tensor,
+        norm_weight: torch.Tensor,
+        eps: float,
+        scale: torch.Tensor = None,
+        x_int_packed: torch.Tensor = None,
+        x_int_row_sum: torch.Tensor = None,
+        x_had: torch.Tensor = None,
+        x_norm: torch.Tensor = None,
+        hadamard_scale: float = HADAMARD_ENTRY,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """RMSNorm (src/models/llama.py:71-77 of the reference) and `hadamard_quantize_int4` of its output in one pass
+    over x (M, K <= 4096): the normalised tensor is not written unless x_norm is given.  Raises RuntimeError with
+    status QUEST_ERR_UNSUPPORTED for longer rows.  Returns (scale, x_int_packed, x_int_row_sum)."""
+    m, k = x.shape
+    assert x.dtype in _FLOAT16S and x.is_contiguous() and norm_weight.dtype == x.dtype and norm_weight.numel() == k
+    assert norm_weight.is_contiguous()
+    scale, x_int_packed, x_int_row_sum = _quant_outputs(m, k, x.dtype, x.device, scale, x_int_packed, x_int_row_sum)
+    for t in (x_had, x_norm):
+        assert t is None or (t.dtype == x.dtype and t.shape == x.shape and t.is_contiguous())
+    dev = require_gpu(x, norm_weight, scale, x_int_packed, x_int_row_sum, x_had, x_norm)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_rmsnorm_hadamard_quantize_int4(
+            ptr(x), ptr(norm_weight), float(eps), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum), ptr(x_had),
+            ptr(x_norm), k, m, float(hadamard_scale), DTYPE_CODE[x.dtype], stream_of(x)), 'rmsnorm_hadamard_quantize_int4')
+    return scale, x_int_packed, x_int_row_sum
+
+
+def silu_mul_hadamard_quantize_int4(
+        gate_up: torch.Tensor,
+        scale: torch.Tensor = None,
+        x_int_packed: torch.Tensor = None,
+        x_int_row_sum: torch.Tensor = None,
+        x_had: torch.Tensor = None,
+        x_act: torch.Tensor = None,
+        hadamard_scale: float = HADAMARD_ENTRY,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """silu(gate) * up (src/models/llama.py:117-118 of the reference) and `hadamard_quantize_int4` of the product in
+    one pass over gate_up (M, 2 K), gate in the first K columns and up in the last K, K <= 4096.  x_act, if given,
+    receives the product (M, K).  Returns (scale, x_int_packed, x_int_row_sum)."""
+    m, k2 = gate_up.shape
+    k = k2 // 2
+    assert gate_up.dtype in _FLOAT16S and gate_up.is_contiguous() and k2 == 2 * k
+    scale, x_int_packed, x_int_row_sum = _quant_outputs(m, k, gate_up.dtype, gate_up.device, scale, x_int_packed, x_int_row_sum)
+    for t in (x_had, x_act):
+        assert t is None or (t.dtype == gate_up.dtype and t.shape == (m, k) and t.is_contiguous())
+    dev = require_gpu(gate_up, scale, x_int_packed, x_int_row_sum, x_had, x_act)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_silu_mul_hadamard_quantize_int4(
+            ptr(gate_up), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum), ptr(x_had), ptr(x_act), k, m,
+            float(hadamard_scale), DTYPE_CODE[gate_up.dtype], stream_of(gate_up)), 'silu_mul_hadamard_quantize_int4')
+    return scale, x_int_packed, x_int_row_sum

@@ -207,9 +207,11 @@ enum { OUT_BF16 = 0, OUT_FP16 = 1, OUT_INT32 = 2 };
 int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                        const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);
 
-// hadamard_mfma.hip: the matrix-core fused activation kernel; QUEST_ERR_UNSUPPORTED when it does not apply
-int launch_hadamard_quantize_mfma(const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had, int K,
-                                  int M, float had_scale, int dtype, hipStream_t st);
+// hadamard_mfma.hip: the matrix-core fused activation kernel, optionally with the producer of the activation in
+// front (pre: 0 none, 1 RMSNorm, 2 SiLU(gate) * up); QUEST_ERR_UNSUPPORTED when it does not apply
+int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
+                                  int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
+                                  hipStream_t st);
 
 inline int check_dtype(int dtype) { return dtype == QUEST_DTYPE_BF16 || dtype == QUEST_DTYPE_FP16; }
 inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

@@ -53,7 +53,7 @@ __device__ __forceinline__ v16f mfma_h(const v4i &a, const v4i &b, const v16f &c
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
-// WPR waves share one row (32 blocks of 128 each); a workgroup holds RPW = max(1, 4 / WPR) rows.
+// WPR waves share one row (32 blocks of 128 each); a workgroup of WPR <= 4 holds 4 / WPR waves' worth of rows.
 template <int WPR>
 struct Shape {
     static constexpr int kRows = WPR >= 4 ? 1 : 4 / WPR;
@@ -61,20 +61,52 @@ struct Shape {
     static constexpr int kMinBlocks = kWaves <= 4 ? 4 : (16 / kWaves > 0 ? 16 / kWaves : 1);
 };
 
-template <int DT, int WPR>
+// What is applied to the input on its way into the transform (the producer the activation comes from):
+//   kPreNone     nothing;
+//   kPreRmsNorm  y = dtype(dtype(f32(x) * rsqrt(mean(x^2) + eps)) * w)    (src/models/llama.py:71-77 of the reference);
+//   kPreSiluMul  y = dtype(dtype(silu(gate)) * up), gate and up the two halves of a (M, 2 K) row (llama.py:117-118).
+enum { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMul = 2 };
+
+// Sum over the G lanes (G a power of two, aligned) of each half-wave that hold one row, and over the two half-waves.
+template <int G>
+__device__ __forceinline__ float group_sum_f(float v) {
+    if constexpr (G >= 2) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+    if constexpr (G >= 4) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+    if constexpr (G >= 8) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+    if constexpr (G >= 16) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));
+    if constexpr (G >= 32) v += lane_xor_f<16>(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <int G>
+__device__ __forceinline__ int group_sum_i(int v) {
+    if constexpr (G >= 2) v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
+    if constexpr (G >= 4) v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
+    if constexpr (G >= 8) v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);
+    if constexpr (G >= 16) v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true);
+    if constexpr (G >= 32) v += lane_xor_i<16>(v);
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+    return (int)r[0] + (int)r[1];
+}
+
+// G = lanes of a half-wave per row (the row's blocks rounded up to a power of two): a wave holds 32 / G rows.
+template <int DT, int WPR, int G, int PRE>
 __global__ void __launch_bounds__(64 * Shape<WPR>::kWaves, Shape<WPR>::kMinBlocks)
-hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ scale, uint32_t *__restrict__ packed,
-                              int32_t *__restrict__ row_sum, uint16_t *__restrict__ x_had, int K, int M,
-                              uint32_t entry_bits) {
+hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ norm_w,
+                              uint16_t *__restrict__ scale, uint32_t *__restrict__ packed, int32_t *__restrict__ row_sum,
+                              uint16_t *__restrict__ x_had, uint16_t *__restrict__ pre_out, int K, int M, int ldx,
+                              uint32_t entry_bits, float eps) {
+    static_assert(WPR == 1 || (G == 32 && PRE == kPreNone), "rows shared by waves: whole waves, no producer");
     constexpr int kRows = Shape<WPR>::kRows;
+    constexpr int kRowsPerWave = 32 / G;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int part = wave % WPR;               // which 32 blocks of the row
     const int row_local = wave / WPR;
-    const int row = blockIdx.x * kRows + row_local;
-    const int n = lane & 31;                   // MFMA column: block 32 part + n of the row
+    const int n = lane & 31;                   // MFMA column
     const int h = lane >> 5;
-    const int blk = part * 32 + n;
+    const int row = (blockIdx.x * kRows + row_local) * kRowsPerWave + n / G;
+    const int blk = part * 32 + n % G;         // block of the row in this column
     const bool live = row < M && blk < (K >> 7);
 
     // ---- the four A fragments: +-entry with sign (-1)^(popcount(n & 7 & j) + n3 h) [* (-1)^n4] [* -1]
@@ -105,11 +137,58 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restri
 
     // ---- B fragments straight from HBM: chunk 2 s + h of a block is bytes [32 s + 16 h, +16) of its 256.
     // Lanes without a block get an offset beyond the buffer: such loads touch no memory and return zeros.
-    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, (int)((long)M * K * 2), 0x00020000);
-    const int ld_off = live ? row * K * 2 + blk * 256 + h * 16 : (int)0x80000000u;
+    const int in_cols = PRE == kPreSiluMul ? 2 * K : K;
+    const __amdgpu_buffer_rsrc_t xr =
+        __builtin_amdgcn_make_buffer_rsrc((void *)x, 0, (int)(((long)(M - 1) * ldx + in_cols) * 2), 0x00020000);
+    const uint32_t dead = 0x80000000u;
+    const uint32_t ld_off = live ? (uint32_t)(row * ldx * 2 + blk * 256 + h * 16) : dead;
     v4u bq[8];
 #pragma unroll
-    for (int s = 0; s < 8; s++) bq[s] = __builtin_amdgcn_raw_buffer_load_b128(xr, ld_off + 32 * s, 0, 0);
+    for (int s = 0; s < 8; s++) bq[s] = __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(ld_off + 32 * s), 0, 0);
+
+    if constexpr (PRE == kPreRmsNorm) {
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, 0x00020000);
+        const uint32_t w_off = live ? (uint32_t)(blk * 256 + h * 16) : dead;
+        v4u wq[8];
+#pragma unroll
+        for (int s = 0; s < 8; s++) wq[s] = __builtin_amdgcn_raw_buffer_load_b128(wr, (int)(w_off + 32 * s), 0, 0);
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int d = 0; d < 4; d++) ss = dot2_self<DT>(bq[s][d], ss);
+        const float mean_sq = __fmul_rn(group_sum_f<G>(ss), __fdiv_rn(1.0f, (float)K));
+        const float r = __frsqrt_rn(__fadd_rn(mean_sq, eps));
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t y = pack2_rounded_products<DT>(__fmul_rn(lo_f32<DT>(bq[s][d]), r), __fmul_rn(hi_f32<DT>(bq[s][d]), r));
+                bq[s][d] = pack2_rounded_products<DT>(__fmul_rn(lo_f32<DT>(y), lo_f32<DT>(wq[s][d])),
+                                                      __fmul_rn(hi_f32<DT>(y), hi_f32<DT>(wq[s][d])));
+            }
+    }
+    if constexpr (PRE == kPreSiluMul) {
+        v4u uq[8];
+#pragma unroll
+        for (int s = 0; s < 8; s++) uq[s] = __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(ld_off + K * 2 + 32 * s), 0, 0);
+        auto silu = [](float g) { return __fdividef(g, 1.0f + __expf(-g)); };
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t a = pack2_rounded_products<DT>(silu(lo_f32<DT>(bq[s][d])), silu(hi_f32<DT>(bq[s][d])));
+                bq[s][d] = pack2_rounded_products<DT>(__fmul_rn(lo_f32<DT>(a), lo_f32<DT>(uq[s][d])),
+                                                      __fmul_rn(hi_f32<DT>(a), hi_f32<DT>(uq[s][d])));
+            }
+    }
+    if constexpr (PRE != kPreNone) {
+        if (pre_out != nullptr && live) {
+            uint16_t *dst = pre_out + (size_t)row * K + blk * 128 + 8 * h;
+#pragma unroll
+            for (int s = 0; s < 8; s++) *reinterpret_cast<v4u *>(dst + 16 * s) = bq[s];
+        }
+    }
 
     // ---- Hadamard: 8 k-steps x 4 row tiles
     v16f acc[4];
@@ -141,7 +220,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restri
                 sumsq = dot2_self<DT>(w, sumsq);            // both squares straight from the packed pair
             }
     // lanes without a block transformed zeros: they add nothing
-    float total = wave_sum_dpp_f(sumsq);
+    float total = G == 32 ? wave_sum_dpp_f(sumsq) : group_sum_f<G>(sumsq);
     __shared__ float part_sq[Shape<WPR>::kWaves];
     __shared__ int part_sum[Shape<WPR>::kWaves];
     if constexpr (WPR > 1) {
@@ -153,6 +232,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restri
     }
     const uint32_t s16 = from_f32<DT>(scale_from_sumsq(total, K));
     const float inv = quant_inv(to_f32<DT>(s16));
+    const bool writer = lane % G == 0 && h == 0 && part == 0 && row < M;      // one lane per row
 
     if (x_had != nullptr && live) {
         uint16_t *dst = x_had + (size_t)row * K + blk * 128 + 4 * h;
@@ -162,7 +242,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restri
             for (int q = 0; q < 4; q++)
                 *reinterpret_cast<uint2 *>(dst + 32 * mt + 8 * q) = make_uint2(yb[mt][q * 2], yb[mt][q * 2 + 1]);
     }
-    if (lane == 0 && part == 0 && row < M) scale[row] = (uint16_t)s16;
+    if (writer) scale[row] = (uint16_t)s16;
     if (packed == nullptr && row_sum == nullptr) return;      // uniform over the workgroup
 
     // ---- codes: c3 c2 c1 c0 (outputs 8 Q + 4 h + {0..3}, Q = 4 mt + q) summed as c_e 16^e: the two's-complement
@@ -199,7 +279,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restri
     }
     if (row_sum != nullptr) {
         if (!live) isum = 0;                    // a dead lane's zeros need not quantise to code 0
-        int t = wave_sum_dpp_i(isum);
+        int t = G == 32 ? wave_sum_dpp_i(isum) : group_sum_i<G>(isum);
         if constexpr (WPR > 1) {
             if (lane == 0) part_sum[wave] = t;
             __syncthreads();
@@ -207,7 +287,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, uint16_t *__restri
 #pragma unroll
             for (int w = 0; w < WPR; w++) t += part_sum[row_local * WPR + w];
         }
-        if (lane == 0 && part == 0 && row < M) row_sum[row] = t;
+        if (writer) row_sum[row] = t;
     }
 }
 
@@ -230,40 +310,79 @@ static bool representable16(float v, int dtype, uint32_t *bits) {
     return true;
 }
 
-template <int DT, int WPR>
-static void launch_shape(const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had, int K, int M,
-                         uint32_t bits, hipStream_t st) {
-    constexpr int kRows = hq::Shape<WPR>::kRows;
-    hq::hadamard_quantize_mfma_kernel<DT, WPR><<<dim3((M + kRows - 1) / kRows), dim3(64 * hq::Shape<WPR>::kWaves), 0, st>>>(
-        (const uint16_t *)x, (uint16_t *)scale, (uint32_t *)packed, row_sum, (uint16_t *)x_had, K, M, bits);
+struct Args {
+    const void *x, *norm_w;
+    void *scale;
+    uint8_t *packed;
+    int32_t *row_sum;
+    void *x_had, *pre_out;
+    int K, M, ldx;
+    uint32_t bits;
+    float eps;
+    hipStream_t st;
+};
+
+template <int DT, int WPR, int G, int PRE>
+static void launch_shape(const Args &a) {
+    constexpr int rows = hq::Shape<WPR>::kRows * (32 / G);        // rows per workgroup
+    hq::hadamard_quantize_mfma_kernel<DT, WPR, G, PRE><<<dim3((a.M + rows - 1) / rows), dim3(64 * hq::Shape<WPR>::kWaves), 0, a.st>>>(
+        (const uint16_t *)a.x, (const uint16_t *)a.norm_w, (uint16_t *)a.scale, (uint32_t *)a.packed, a.row_sum,
+        (uint16_t *)a.x_had, (uint16_t *)a.pre_out, a.K, a.M, a.ldx, a.bits, a.eps);
 }
 
-template <int DT>
-static void launch_dtype(int wpr, const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had, int K,
-                         int M, uint32_t bits, hipStream_t st) {
-    switch (wpr) {
-        case 1: launch_shape<DT, 1>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        case 2: launch_shape<DT, 2>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        case 3: launch_shape<DT, 3>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        case 4: launch_shape<DT, 4>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        case 5: launch_shape<DT, 5>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        case 6: launch_shape<DT, 6>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        case 7: launch_shape<DT, 7>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
-        default: launch_shape<DT, 8>(x, scale, packed, row_sum, x_had, K, M, bits, st); break;
+// rows of up to 32 blocks: one wave holds 32 / G of them
+template <int DT, int PRE>
+static void launch_short(int g, const Args &a) {
+    switch (g) {
+        case 1: launch_shape<DT, 1, 1, PRE>(a); break;
+        case 2: launch_shape<DT, 1, 2, PRE>(a); break;
+        case 4: launch_shape<DT, 1, 4, PRE>(a); break;
+        case 8: launch_shape<DT, 1, 8, PRE>(a); break;
+        case 16: launch_shape<DT, 1, 16, PRE>(a); break;
+        default: launch_shape<DT, 1, 32, PRE>(a); break;
     }
 }
 
-// Launches the matrix-core kernel when it applies (K a multiple of 128 up to 32768, a Hadamard entry the
-// dtype represents exactly); returns QUEST_ERR_UNSUPPORTED otherwise so that the caller takes the butterfly kernel.
-int launch_hadamard_quantize_mfma(const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had, int K,
-                                  int M, float had_scale, int dtype, hipStream_t st) {
+// longer rows: WPR waves per row
+template <int DT>
+static void launch_long(int wpr, const Args &a) {
+    switch (wpr) {
+        case 2: launch_shape<DT, 2, 32, hq::kPreNone>(a); break;
+        case 3: launch_shape<DT, 3, 32, hq::kPreNone>(a); break;
+        case 4: launch_shape<DT, 4, 32, hq::kPreNone>(a); break;
+        case 5: launch_shape<DT, 5, 32, hq::kPreNone>(a); break;
+        case 6: launch_shape<DT, 6, 32, hq::kPreNone>(a); break;
+        case 7: launch_shape<DT, 7, 32, hq::kPreNone>(a); break;
+        default: launch_shape<DT, 8, 32, hq::kPreNone>(a); break;
+    }
+}
+
+template <int DT>
+static void launch_dtype(int pre, const Args &a) {
+    const int nb = a.K / 128;
+    if (nb > 32) return launch_long<DT>((nb + 31) / 32, a);
+    int g = 1;
+    while (g < nb) g *= 2;
+    if (pre == hq::kPreRmsNorm) launch_short<DT, hq::kPreRmsNorm>(g, a);
+    else if (pre == hq::kPreSiluMul) launch_short<DT, hq::kPreSiluMul>(g, a);
+    else launch_short<DT, hq::kPreNone>(g, a);
+}
+
+// Launches the matrix-core kernel when it applies (K a multiple of 128 up to 32768 -- 4096 with a producer --, a
+// Hadamard entry the dtype represents exactly); returns QUEST_ERR_UNSUPPORTED otherwise so that the caller can take
+// another path.  pre: 0 none, 1 RMSNorm (norm_w, eps), 2 SiLU(gate) * up with x a (M, 2 K) tensor.
+int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
+                                  int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
+                                  hipStream_t st) {
     uint32_t bits = 0;
     if (K > 32768 || (K & 127) || had_scale <= 0.f || !representable16(had_scale, dtype, &bits)) return QUEST_ERR_UNSUPPORTED;
-    if ((long)M * K * 2 >= (1L << 31)) return QUEST_ERR_UNSUPPORTED;          // 32-bit buffer offsets
-    if (!aligned(packed, 16) || !aligned(x_had, 8)) return QUEST_ERR_UNSUPPORTED;
-    const int wpr = (K / 128 + 31) / 32;       // waves per row
-    if (dtype == QUEST_DTYPE_BF16) launch_dtype<0>(wpr, x, scale, packed, row_sum, x_had, K, M, bits, st);
-    else launch_dtype<1>(wpr, x, scale, packed, row_sum, x_had, K, M, bits, st);
+    if (pre != hq::kPreNone && K > 4096) return QUEST_ERR_UNSUPPORTED;
+    const int ldx = pre == hq::kPreSiluMul ? 2 * K : K;
+    if ((long)M * ldx * 2 >= (1L << 31)) return QUEST_ERR_UNSUPPORTED;        // 32-bit buffer offsets
+    if (!aligned(packed, 16) || !aligned(x_had, 8) || !aligned(pre_out, 16) || !aligned(norm_w, 16)) return QUEST_ERR_UNSUPPORTED;
+    const Args a = {x, norm_w, scale, packed, row_sum, x_had, pre_out, K, M, ldx, bits, eps, st};
+    if (dtype == QUEST_DTYPE_BF16) launch_dtype<0>(pre, a);
+    else launch_dtype<1>(pre, a);
     return launch_status();
 }
 

@@ -351,10 +351,34 @@ extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t 
     if (!aligned(x, 16) || !aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
     hipStream_t st = (hipStream_t)stream;
     // rows of up to 32768 with a Hadamard entry the dtype holds exactly: matrix cores; anything else: butterflies
-    const int rc = launch_hadamard_quantize_mfma(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size,
-                                                 had_scale, dtype, st);
+    const int rc = launch_hadamard_quantize_mfma(0, x, nullptr, 0.f, scale, x_int_packed, x_int_row_sum, x_had, nullptr,
+                                                 group_size, batch_size, had_scale, dtype, st);
     if (rc != QUEST_ERR_UNSUPPORTED) return rc;
     if (dtype == QUEST_DTYPE_BF16)
         return launch_hadamard_quantize<0>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale, st);
     return launch_hadamard_quantize<1>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale, st);
+}
+
+extern "C" int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *norm_weight, float eps, void *scale,
+                                                    uint8_t *x_int_packed, int32_t *x_int_row_sum, void *x_had,
+                                                    void *x_norm, int group_size, int batch_size, float had_scale,
+                                                    int dtype, void *stream) {
+    if (!x || !norm_weight || !scale) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(x, 16) || !aligned(norm_weight, 16) || !aligned(x_had, 16) || !aligned(x_norm, 16) || !aligned(x_int_packed, 16))
+        return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(1, x, norm_weight, eps, scale, x_int_packed, x_int_row_sum, x_had, x_norm,
+                                         group_size, batch_size, had_scale, dtype, (hipStream_t)stream);
+}
+
+extern "C" int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *scale, uint8_t *x_int_packed,
+                                                     int32_t *x_int_row_sum, void *x_had, void *x_act, int group_size,
+                                                     int batch_size, float had_scale, int dtype, void *stream) {
+    if (!gate_up || !scale) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(gate_up, 16) || !aligned(x_had, 16) || !aligned(x_act, 16) || !aligned(x_int_packed, 16)) return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(2, gate_up, nullptr, 0.f, scale, x_int_packed, x_int_row_sum, x_had, x_act,
+                                         group_size, batch_size, had_scale, dtype, (hipStream_t)stream);
 }

@@ -206,7 +206,8 @@ def test_hadamard128(quest, dtype, scale):
 # --------------------------------------------------------------------------- fused activation kernel
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768), (64, 4096), (1, 128), (8, 11008), (16, 2816), (2, 16384), (2, 32768),
-                                   (3, 1024), (777, 4096), (5, 3968), (3, 5120), (6, 8192), (2, 28672), (2, 65536)])
+                                   (3, 1024), (777, 4096), (5, 3968), (3, 5120), (6, 8192), (2, 28672), (2, 65536),
+                                   (50, 256), (50, 512), (37, 2048), (130, 1024), (70, 128)])
 def test_hadamard_quantize_fused(quest, dtype, shape):
     """Rows of up to 32768 run the Hadamard on the matrix cores (the reference's matmul formulation, fp32
     accumulation in the hardware's order; rows over 4096 are shared by the waves of a workgroup), longer
@@ -263,6 +264,69 @@ def test_hadamard_quantize_weight_scale_runs_butterflies(quest, dtype):
     rs = torch.empty(96, 1, dtype=torch.int32)
     qo.quantize_int4(want_had.clone(), scale.cpu(), None, xp, rs, False)
     assert torch.equal(packed.cpu(), xp) and torch.equal(row_sum.cpu(), rs)
+
+
+# --------------------------------------------------------------------------- producers fused in front
+def _ulp_stats(got, want):
+    d = ulp_diff(got, want)
+    return int(d.max()), float((d != 0).float().mean())
+
+
+PRODUCER_SHAPES = [(160, 1024), (33, 2816), (5, 128), (64, 4096), (7, 256), (9, 512), (12, 2048), (300, 768)]
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', PRODUCER_SHAPES)
+def test_rmsnorm_hadamard_quantize(quest, dtype, shape):
+    """RMSNorm in front of the fused kernel.  The normalised tensor agrees with torch's CPU RMSNorm up to the last
+    bit of a few elements (fp32 reduction order and rsqrt), and from that tensor on the kernel is the plain fused
+    kernel bit for bit."""
+    from oracle import llama_oracle as lo
+    m, k = shape
+    x = rand_act(m, k, dtype, seed=20)
+    w = (1 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(21))).to(dtype)
+    gx, gw = x.to(DEV), w.to(DEV)
+    x_norm = torch.empty_like(gx)
+    x_had = torch.empty_like(gx)
+    scale, packed, row_sum = quest.rmsnorm_hadamard_quantize_int4(gx, gw, 1e-5, x_had=x_had, x_norm=x_norm)
+    assert torch.equal(bits(gx.cpu()), bits(x)), 'input must not be written'
+    worst, frac = _ulp_stats(x_norm.cpu(), lo.rmsnorm(x, w, 1e-5))
+    assert worst <= 2 and frac < 0.02, (worst, frac)
+    had2 = torch.empty_like(gx)
+    s2, p2, r2 = quest.hadamard_quantize_int4(x_norm, x_had=had2)
+    assert torch.equal(bits(x_had.cpu()), bits(had2.cpu()))
+    assert torch.equal(bits(scale.cpu()), bits(s2.cpu())) and torch.equal(packed, p2) and torch.equal(row_sum, r2)
+    # outputs that are not asked for
+    s3, p3, r3 = quest.rmsnorm_hadamard_quantize_int4(gx, gw, 1e-5)
+    assert torch.equal(bits(s3.cpu()), bits(scale.cpu())) and torch.equal(p3, packed) and torch.equal(r3, row_sum)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', PRODUCER_SHAPES)
+def test_silu_mul_hadamard_quantize(quest, dtype, shape):
+    """SwiGLU product in front of the fused kernel, against torch's CPU silu(gate) * up."""
+    m, k = shape
+    gu = rand_act(m, 2 * k, dtype, seed=22)
+    want = torch.nn.functional.silu(gu[:, :k]) * gu[:, k:]
+    ggu = gu.to(DEV)
+    x_act = torch.empty(m, k, dtype=dtype, device=DEV)
+    x_had = torch.empty_like(x_act)
+    scale, packed, row_sum = quest.silu_mul_hadamard_quantize_int4(ggu, x_had=x_had, x_act=x_act)
+    assert torch.equal(bits(ggu.cpu()), bits(gu)), 'input must not be written'
+    worst, frac = _ulp_stats(x_act.cpu(), want)
+    assert worst <= 2 and frac < 0.02, (worst, frac)
+    had2 = torch.empty_like(x_act)
+    s2, p2, r2 = quest.hadamard_quantize_int4(x_act, x_had=had2)
+    assert torch.equal(bits(x_had.cpu()), bits(had2.cpu()))
+    assert torch.equal(bits(scale.cpu()), bits(s2.cpu())) and torch.equal(packed, p2) and torch.equal(row_sum, r2)
+
+
+def test_producers_refuse_long_rows(quest):
+    x = torch.zeros(2, 8192, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        quest.rmsnorm_hadamard_quantize_int4(x, torch.ones(8192, dtype=torch.bfloat16, device=DEV), 1e-5)
+    with pytest.raises(RuntimeError):
+        quest.silu_mul_hadamard_quantize_int4(torch.zeros(2, 16384, dtype=torch.bfloat16, device=DEV))
 
 
 def test_hadamard_quantize_is_deterministic(quest):
