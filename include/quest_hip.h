@@ -134,6 +134,18 @@ int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *scale, uint
                                           int32_t *x_int_row_sum, void *x_had, void *x_act, int group_size,
                                           int batch_size, float had_scale, int dtype, void *stream);
 
+/*
+ * Rotary position embedding, in place, on the first rot_cols elements of each of n_rows rows of x (row pitch
+ * row_stride elements): the columns are heads of head_dim elements holding interleaved (re, im) pairs; row r is
+ * position r % seq_len; freqs_cis is fp32 (seq_len, head_dim / 2, 2) = (cos, sin).  out_re = re cos - im sin,
+ * out_im = re sin + im cos, every product and sum rounded to fp32, one rounding to dtype: bit for bit what
+ * apply_rotary_emb (src/models/llama.py:43-62) computes for q and k.  With x the (B T, 3 d) output of the fused
+ * QKV projection and rot_cols = 2 d it rotates q and k where they lie and leaves v alone.
+ * head_dim % 8 == 0, rot_cols % head_dim == 0, row_stride % 8 == 0.
+ */
+int quest_rope_interleaved(void *x, const float *freqs_cis, int n_rows, int seq_len, int row_stride,
+                           int rot_cols, int head_dim, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -260,3 +260,17 @@ def silu_mul_hadamard_quantize_int4(
             ptr(gate_up), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum), ptr(x_had), ptr(x_act), k, m,
             float(hadamard_scale), DTYPE_CODE[gate_up.dtype], stream_of(gate_up)), 'silu_mul_hadamard_quantize_int4')
     return scale, x_int_packed, x_int_row_sum
+
+
+def rope_interleaved_(x: torch.Tensor, freqs_cis: torch.Tensor, rot_cols: int, head_dim: int) -> torch.Tensor:
+    """In-place rotary embedding of the first rot_cols columns of x (B, T, C) (src/models/llama.py:43-62 of the
+    reference, for q and k at once when x is the fused QKV projection and rot_cols = 2 d).  freqs_cis: fp32
+    (T, head_dim / 2, 2)."""
+    b, t, c = x.shape
+    assert x.dtype in _FLOAT16S and x.is_contiguous()
+    assert freqs_cis.dtype == torch.float32 and freqs_cis.is_contiguous() and freqs_cis.shape == (t, head_dim // 2, 2)
+    dev = require_gpu(x, freqs_cis)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_rope_interleaved(ptr(x), ptr(freqs_cis), b * t, t, c, rot_cols, head_dim,
+                                                 DTYPE_CODE[x.dtype], stream_of(x)), 'rope_interleaved')
+    return x

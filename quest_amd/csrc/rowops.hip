@@ -272,6 +272,38 @@ static int launch_hadamard_quantize(const void *x, void *scale, uint8_t *packed,
     return launch_status();
 }
 
+// Rotary position embedding on interleaved pairs, in place (src/models/llama.py:43-62 of the reference): the first
+// n_heads * head_dim elements of every row are heads of (re, im) pairs; pair i of a head at position t turns by the
+// angle whose (cos, sin) is freqs[t][i].  fp32 products and sums in the reference's order, one rounding to dtype.
+template <int DT>
+__global__ void __launch_bounds__(256)
+rope_kernel(uint16_t *__restrict__ x, const float *__restrict__ freqs, int n_rows, int seq_len, int row_stride,
+            int rot_cols, int head_dim) {
+    const int chunks = rot_cols >> 3;                        // 16-byte chunks (4 pairs) to rotate per row
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long)n_rows * chunks) return;
+    const int row = (int)(idx / chunks);
+    const int col = (int)(idx % chunks) * 8;
+    const int t = row % seq_len;
+    const int pair0 = (col % head_dim) >> 1;
+    uint4 *p = reinterpret_cast<uint4 *>(x + (size_t)row * row_stride + col);
+    const float4 *f = reinterpret_cast<const float4 *>(freqs + ((size_t)t * (head_dim >> 1) + pair0) * 2);
+    const uint4 v = *p;
+    const float4 f01 = f[0], f23 = f[1];
+    const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+    const float cs[4][2] = {{f01.x, f01.y}, {f01.z, f01.w}, {f23.x, f23.y}, {f23.z, f23.w}};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float re = lo_f32<DT>(in[i]), im = hi_f32<DT>(in[i]);
+        const float c = cs[i][0], sn = cs[i][1];
+        const float out_re = __fsub_rn(__fmul_rn(re, c), __fmul_rn(im, sn));
+        const float out_im = __fadd_rn(__fmul_rn(re, sn), __fmul_rn(im, c));
+        o[i] = from_f32<DT>(out_re) | (from_f32<DT>(out_im) << 16);
+    }
+    *p = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 }  // namespace quest
 
 using namespace quest;
@@ -381,4 +413,22 @@ extern "C" int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *
     if (!aligned(gate_up, 16) || !aligned(x_had, 16) || !aligned(x_act, 16) || !aligned(x_int_packed, 16)) return QUEST_ERR_ALIGNMENT;
     return launch_hadamard_quantize_mfma(2, gate_up, nullptr, 0.f, scale, x_int_packed, x_int_row_sum, x_had, x_act,
                                          group_size, batch_size, had_scale, dtype, (hipStream_t)stream);
+}
+
+extern "C" int quest_rope_interleaved(void *x, const float *freqs_cis, int n_rows, int seq_len, int row_stride,
+                                      int rot_cols, int head_dim, int dtype, void *stream) {
+    if (!x || !freqs_cis) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (n_rows <= 0 || seq_len <= 0 || rot_cols <= 0 || head_dim <= 0 || (head_dim & 7) || (rot_cols % head_dim) ||
+        rot_cols > row_stride || (row_stride & 7))
+        return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(x, 16) || !aligned(freqs_cis, 16)) return QUEST_ERR_ALIGNMENT;
+    const long work = (long)n_rows * (rot_cols >> 3);
+    const unsigned blocks = (unsigned)((work + 255) / 256);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == QUEST_DTYPE_BF16)
+        rope_kernel<0><<<dim3(blocks), dim3(256), 0, st>>>((uint16_t *)x, freqs_cis, n_rows, seq_len, row_stride, rot_cols, head_dim);
+    else
+        rope_kernel<1><<<dim3(blocks), dim3(256), 0, st>>>((uint16_t *)x, freqs_cis, n_rows, seq_len, row_stride, rot_cols, head_dim);
+    return launch_status();
 }

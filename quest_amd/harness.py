@@ -172,6 +172,16 @@ class Linear4bit(nn.Module):
         self.register_buffer('w_meta_e', None)
         return self
 
+    def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None) -> torch.Tensor:
+        """The GEMM half of `linear_forward` on activations some fused producer kernel has already quantised:
+        (M, 1) scales, (M, K/2) codes, (M, 1) row sums -> (M, N)."""
+        y = quest.fused_matmul_dequantize_int4_int4t_bf16(mat_a=a_int_packed, mat_b=self.w_int_packed,
+                                                          vec_a_add=a_int_row_sum, vec_b_add=self.w_add,
+                                                          vec_a_mul=a_scale, vec_b_mul=self.w_scale, out=out)
+        if self.bias is not None:
+            y += self.bias
+        return y
+
     def forward(self, x) -> torch.Tensor:
         if not self.use_noop:
             a = x.contiguous().flatten(end_dim=-2)

@@ -12,7 +12,8 @@ Modes (bench_e2e.py:84-95): 'bf16' dense torch linears, 'int4' packed INT4 weigh
 'noop' the same modules returning zeros (everything but the linears).  Two things differ from the reference's
 'int4' wiring, both switchable: gate and up projections (`w1`, `w2`) read the same tensor, so it is quantised
 once and multiplied by the concatenated weights in one GEMM (`fuse_gate_up`); the reference launches them
-separately (llama.py:89-106, 117-118).
+separately (llama.py:89-106, 117-118); and with `fuse_producers` the RMSNorms and the SwiGLU product run inside
+the quantising kernels of the linears they feed.
 """
 from __future__ import annotations
 
@@ -23,6 +24,7 @@ import torch
 from torch import nn
 from torch.nn import functional as F
 
+from . import api as quest
 from . import harness
 
 
@@ -113,10 +115,22 @@ class LlamaAttention(nn.Module):
         self.c_attn = nn.Linear(config.n_embd, 3 * config.n_embd, bias=config.bias)
         self.c_proj = nn.Linear(config.n_embd, config.n_embd, bias=config.bias)
         self.n_head, self.n_embd = config.n_head, config.n_embd
+        self.fused_rope = False          # set by quantize_model(..., fuse_producers=True)
 
     def forward(self, x, freqs_cis):
-        b, t, c = x.size()
-        q, k, v = self.c_attn(x).split(self.n_embd, dim=2)
+        return self.attend(self.c_attn(x), freqs_cis)
+
+    def attend(self, qkv, freqs_cis):
+        """Everything after the QKV projection: qkv (B, T, 3 d) -> (B, T, d)."""
+        b, t, c3 = qkv.size()
+        c = c3 // 3
+        if self.fused_rope and qkv.is_cuda and qkv.is_contiguous():
+            # q and k rotated where they lie in the projection's output (one kernel, bit-identical to apply_rotary_emb)
+            quest.rope_interleaved_(qkv, freqs_cis.contiguous(), 2 * c, c // self.n_head)
+            q, k, v = (z.view(b, t, self.n_head, c // self.n_head).transpose(1, 2) for z in qkv.split(self.n_embd, dim=2))
+            y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=True)
+            return self.c_proj(y.transpose(1, 2).contiguous().view(b, t, c))
+        q, k, v = qkv.split(self.n_embd, dim=2)
         k = k.view(b, t, self.n_head, c // self.n_head)
         q = q.view(b, t, self.n_head, c // self.n_head)
         q, k = apply_rotary_emb(q, k, freqs_cis)
@@ -136,9 +150,27 @@ class LlamaBlock(nn.Module):
         self.ln_2 = RMSNorm(config.n_embd, eps=config.rmsnorm_eps)
         self.mlp = LlamaMLP(config)
 
+        self.fuse_producers = False      # set by quantize_model: norms and SwiGLU product folded into the quantiser
+
     def forward(self, x, freqs_cis):
+        if self.fuse_producers:
+            return self._forward_fused(x, freqs_cis)
         x = x + self.attn(self.ln_1(x), freqs_cis)
         return x + self.mlp(self.ln_2(x))
+
+    def _forward_fused(self, x, freqs_cis):
+        """The same block with each W4A4 linear fed by the kernel that also computes its input: RMSNorm -> codes for
+        c_attn and for the fused gate/up projection, silu(gate) * up -> codes for the MLP's c_proj.  Three bf16
+        tensors per block (two normalised activations, one SwiGLU product) are never written or re-read."""
+        b, t, c = x.shape
+        x2 = x.view(b * t, c)
+        q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
+        x = x + self.attn.attend(self.attn.c_attn.forward_quantized(*q).view(b, t, 3 * c), freqs_cis)
+        x2 = x.view(b * t, c)
+        q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_2.weight, self.ln_2.eps)
+        gate_up = self.mlp.w12.forward_quantized(*q)
+        q = quest.silu_mul_hadamard_quantize_int4(gate_up)
+        return x + self.mlp.c_proj.forward_quantized(*q).view(b, t, c)
 
 
 class Llama(nn.Module):
@@ -194,7 +226,8 @@ def _pack(linear: nn.Linear, use_hadamard: bool, use_noop: bool) -> harness.Line
 
 
 @torch.no_grad()
-def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, fuse_gate_up: bool = True) -> Llama:
+def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, fuse_gate_up: bool = True,
+                   fuse_producers: bool = False) -> Llama:
     """bench_e2e.py:77-97 on an existing model: every linear under `transformer` becomes a `Linear4bit` holding the
     packed INT4 form of that linear's own weight ('int4'), or the same module in no-op mode ('noop'); 'bf16' leaves
     the dense linears.  The model must already sit on the GPU in bf16 or fp16."""
@@ -217,6 +250,10 @@ def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, 
             mlp.w1 = _pack(mlp.w1, use_hadamard, noop)
             mlp.w2 = _pack(mlp.w2, use_hadamard, noop)
         mlp.c_proj = _pack(mlp.c_proj, use_hadamard, noop)
+        # the producer-fused kernels exist for the Hadamard variant, rows up to 4096 and the fused gate/up layout
+        block.attn.fused_rope = bool(fuse_producers and not noop)
+        block.fuse_producers = bool(fuse_producers and not noop and use_hadamard and fuse_gate_up and
+                                    model.config.n_embd <= 4096 and model.config.hidden_dim <= 4096)
     return model
 
 

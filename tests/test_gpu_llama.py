@@ -94,9 +94,28 @@ def test_fused_gate_up_is_bit_identical_to_separate(llama):
     assert torch.equal(ya, yb)
 
 
+def test_fused_producers_track_the_unfused_model(llama):
+    """RMSNorm and SwiGLU folded into the quantising kernels: their intermediate tensors match torch's to the last
+    bit of a few elements (tested per kernel), which flips a few codes, so logits agree to INT4-noise level only;
+    far closer to the unfused INT4 model than that model is to the dense one."""
+    a, cfg, weights = build(llama, torch.bfloat16, seed=7)
+    b, _, _ = build(llama, torch.bfloat16, seed=7)
+    llama.quantize_model(a, 'int4', use_hadamard=True, fuse_gate_up=True, fuse_producers=True)
+    llama.quantize_model(b, 'int4', use_hadamard=True, fuse_gate_up=True, fuse_producers=False)
+    assert all(blk.fuse_producers for blk in a.transformer.h) and not any(blk.fuse_producers for blk in b.transformer.h)
+    ids = torch.randint(0, cfg.vocab_size, (2, 48), generator=torch.Generator().manual_seed(8))
+    dense = lo.forward(weights, ids, cfg.n_layer, cfg.n_head, cfg.rmsnorm_eps, linear='dense').double()
+    with torch.no_grad():
+        ya = a(ids.to(DEV), all_logits=True)['logits'].double().cpu()
+        yb = b(ids.to(DEV), all_logits=True)['logits'].double().cpu()
+    err = (ya - yb).norm() / yb.norm()
+    gap = (yb - dense).norm() / dense.norm()
+    assert err < 0.5 * gap, (float(err), float(gap))
+
+
 def test_graph_replay_and_noop(llama):
     model, cfg, _ = build(llama, torch.bfloat16, seed=4)
-    llama.quantize_model(model, 'int4', use_hadamard=True)
+    llama.quantize_model(model, 'int4', use_hadamard=True, fuse_producers=True)
     r = llama.bench_forward(model, batch_size=2, seq_len=32, n_warmup=2, n_iter=2)
     assert r['graph_matches_eager'] and r['best_s'] > 0
     noop, _, _ = build(llama, torch.bfloat16, seed=4)

@@ -329,6 +329,25 @@ def test_producers_refuse_long_rows(quest):
         quest.silu_mul_hadamard_quantize_int4(torch.zeros(2, 16384, dtype=torch.bfloat16, device=DEV))
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(2, 48, 4, 64), (3, 17, 2, 32), (1, 512, 16, 64), (2, 5, 1, 8)])
+def test_rope_in_place_bit_exact(quest, dtype, shape):
+    """q and k rotated inside a fused QKV tensor, against the reference's formulation on the CPU; v untouched."""
+    from oracle import llama_oracle as lo
+    b, t, nh, hs = shape
+    d = nh * hs
+    g = torch.Generator().manual_seed(30)
+    qkv = torch.randn(b, t, 3 * d, generator=g).to(dtype)
+    fc = lo.precompute_freqs_cis(hs, t)
+    q, k, v = qkv.split(d, dim=2)
+    want_q, want_k = lo.apply_rotary_emb(q.reshape(b, t, nh, hs), k.reshape(b, t, nh, hs), fc)
+    got = quest.rope_interleaved_(qkv.to(DEV), fc.to(DEV), 2 * d, hs).cpu()
+    gq, gk, gv = got.split(d, dim=2)
+    assert torch.equal(bits(gq.reshape(b, t, nh, hs)), bits(want_q))
+    assert torch.equal(bits(gk.reshape(b, t, nh, hs)), bits(want_k))
+    assert torch.equal(bits(gv.contiguous()), bits(v.contiguous()))
+
+
 def test_hadamard_quantize_is_deterministic(quest):
     x = rand_act(512, 4096, torch.bfloat16, seed=12).to(DEV)
     a = quest.hadamard_quantize_int4(x)
