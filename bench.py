@@ -224,7 +224,7 @@ def bench_forward(dev):
     out = {}
     cfg = llama.LlamaConfig()
     batch, seq = 32, cfg.sequence_length
-    for mode in ('bf16', 'int4', 'int4_fused_producers', 'noop'):
+    for mode in ('bf16', 'bf16_fused_producers', 'int4', 'int4_fused_producers', 'noop'):
         torch.manual_seed(0)
         model = llama.Llama(cfg).to(torch.bfloat16).to(dev).eval()
         llama.quantize_model(model, mode.split('_')[0], use_hadamard=True, fuse_gate_up=True,
@@ -239,6 +239,7 @@ def bench_forward(dev):
     return {'model': '12 layers, d=1024, 16 heads, SwiGLU 2816, vocab 32000, random init', 'tokens': batch * seq,
             'modes': out, 'int4_tokens_per_s': batch * seq / (out['int4_fused_producers']['best_ms'] * 1e-3),
             'speedup_over_bf16': out['bf16']['best_ms'] / out['int4_fused_producers']['best_ms'],
+            'speedup_over_bf16_with_rotary_kernel': out['bf16_fused_producers']['best_ms'] / out['int4_fused_producers']['best_ms'],
             'linear_int_ops': ops, 'linear_ms': lin_ms,
             'linear_frac_of_int8_peak': ops / (lin_ms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS,
             'wiring': 'QKV fused (as the reference); gate and up share one quantisation and one GEMM'}

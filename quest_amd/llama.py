@@ -232,6 +232,8 @@ def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, 
     packed INT4 form of that linear's own weight ('int4'), or the same module in no-op mode ('noop'); 'bf16' leaves
     the dense linears.  The model must already sit on the GPU in bf16 or fp16."""
     if mode == 'bf16':
+        for block in model.transformer.h:          # dense linears; only the rotary kernel replaces torch glue
+            block.attn.fused_rope = bool(fuse_producers)
         return model
     if mode not in ('int4', 'noop'):
         raise NotImplementedError(mode)
