@@ -66,15 +66,7 @@ def load_llama(path: str, device) -> Llama:
 def _skeleton(config: LlamaConfig, dtype, device, use_hadamard: bool, fuse_gate_up: bool) -> Llama:
     """The module tree of a packed model with unset storage: dense parts on `device` in `dtype`, linears as empty
     `Linear4bit`."""
-    saved = torch.nn.Linear.reset_parameters, torch.nn.Embedding.reset_parameters
-    torch.nn.Linear.reset_parameters = lambda self: None
-    torch.nn.Embedding.reset_parameters = lambda self: None
-    try:
-        with torch.device(device):
-            small = LlamaConfig(**{**asdict(config), 'n_layer': 0})
-            model = Llama(small).to(dtype)
-    finally:
-        torch.nn.Linear.reset_parameters, torch.nn.Embedding.reset_parameters = saved
+    model = Llama(LlamaConfig(**{**asdict(config), 'n_layer': 0})).to(device=device, dtype=dtype)   # embeddings, final norm, lm_head
     model.config = config
     d, h = config.n_embd, config.hidden_dim
     mk = lambda i, o: harness.Linear4bit.empty(i, o, bias=config.bias, device=device, dtype=dtype,   # noqa: E731
