@@ -20,6 +20,7 @@ are converted).  The JSON line also carries
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -48,17 +49,32 @@ def mean_ms(pairs):
     return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
 
 
+def current_stream():
+    """torch's current HIP stream as the C ABI takes it; read at every launch so that a capturing stream is honoured."""
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
 def launches_ms(launch, n, warmup=5):
-    """Average duration of `n` back-to-back launches of one kernel: HIP events on torch's current stream (the
-    stream the launches are given) around the whole batch.  `launch(i)` must be a bare C-ABI call, cheap enough
-    on the host that the queue never runs dry; gaps between kernels count as kernel time."""
+    """Average duration of `n` back-to-back launches of one kernel: HIP events on the stream the launches go to,
+    around one replay of a HIP graph that holds the whole batch (a graph keeps the gap between two dispatches to a
+    fraction of a microsecond; whatever gap remains counts as kernel time).  `launch(i)` must be a bare C-ABI call
+    that reads torch's current stream at call time."""
     for i in range(warmup):
         launch(i)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(n):
+                launch(i)
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()                               # once untimed
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     a.record()
-    for i in range(n):
-        launch(i)
+    graph.replay()
     b.record()
     torch.cuda.synchronize()
     return a.elapsed_time(b) / n
@@ -117,7 +133,6 @@ def bench_linear(quest, _lib, steps, warmup, dev):
     # the GEMM alone, bare C-ABI launches: on uniform random activation codes (the stated GEMM workload; the
     # matrix cores draw the most power on them) and on the codes the last step left (Gaussian activations)
     lib = _lib.load()
-    st = _lib.stream_of(out)
     u_codes = torch.randint(-8, 8, (m, k), generator=g, dtype=torch.int8)
     u_packed = ((u_codes[:, 1::2] << 4) | (u_codes[:, ::2] & 0xF)).view(torch.uint8).to(dev)
     u_row_sum = u_codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32).to(dev)
@@ -125,10 +140,10 @@ def bench_linear(quest, _lib, steps, warmup, dev):
 
     def gemm_launcher(codes, row_sum, scale):
         args = (_lib.ptr(out), _lib.ptr(codes), _lib.ptr(w_packed), _lib.ptr(row_sum), _lib.ptr(w_add),
-                _lib.ptr(scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype], st)     # sizes in the ABI's order: M, K, N
+                _lib.ptr(scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype])         # sizes in the ABI's order: M, K, N
 
         def gemm(_):
-            if lib.quest_fused_matmul_dequantize_int4_int4t(*args) != 0:
+            if lib.quest_fused_matmul_dequantize_int4_int4t(*args, current_stream()) != 0:
                 raise RuntimeError('GEMM launch failed')
         return gemm
 
@@ -156,12 +171,11 @@ def bench_quantize(_lib, steps, warmup, dev):
     packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
     row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
     lib = _lib.load()
-    st = _lib.stream_of(scale)
     xp = [_lib.ptr(x) for x in xs]
-    tail = (_lib.ptr(scale), _lib.ptr(packed), _lib.ptr(row_sum), None, k, m, 181. / 2048., _lib.DTYPE_CODE[dtype], st)
+    tail = (_lib.ptr(scale), _lib.ptr(packed), _lib.ptr(row_sum), None, k, m, 181. / 2048., _lib.DTYPE_CODE[dtype])
 
     def launch(i):
-        if lib.quest_hadamard_quantize_int4(xp[i % n_buf], *tail) != 0:
+        if lib.quest_hadamard_quantize_int4(xp[i % n_buf], *tail, current_stream()) != 0:
             raise RuntimeError('activation kernel launch failed')
 
     ms = launches_ms(launch, steps, warmup)
@@ -191,18 +205,17 @@ def bench_decode(_lib, dev):
             a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
             a_row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
             y = torch.empty(m, n, dtype=dtype, device=dev)
-            st = _lib.stream_of(y)
-            q_args = (_lib.ptr(x), _lib.ptr(a_scale), _lib.ptr(a_packed), _lib.ptr(a_row_sum), None, k, m, 181. / 2048., code, st)
+            q_args = (_lib.ptr(x), _lib.ptr(a_scale), _lib.ptr(a_packed), _lib.ptr(a_row_sum), None, k, m, 181. / 2048., code)
             wp = [_lib.ptr(w) for w in ws]
-            g_tail = (_lib.ptr(a_row_sum), _lib.ptr(w_add), _lib.ptr(a_scale), _lib.ptr(w_scale), m, k, n, code, st)
+            g_tail = (_lib.ptr(a_row_sum), _lib.ptr(w_add), _lib.ptr(a_scale), _lib.ptr(w_scale), m, k, n, code)
             yp, ap = _lib.ptr(y), _lib.ptr(a_packed)
 
             def gemm(i):
-                if lib.quest_fused_matmul_dequantize_int4_int4t(yp, ap, wp[i % n_w], *g_tail) != 0:
+                if lib.quest_fused_matmul_dequantize_int4_int4t(yp, ap, wp[i % n_w], *g_tail, current_stream()) != 0:
                     raise RuntimeError('GEMM launch failed')
 
             def layer(i):
-                if lib.quest_hadamard_quantize_int4(*q_args) != 0:
+                if lib.quest_hadamard_quantize_int4(*q_args, current_stream()) != 0:
                     raise RuntimeError('activation kernel launch failed')
                 gemm(i)
 
