@@ -111,6 +111,17 @@ int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t *x_int_pack
                                  float had_scale, int dtype, void *stream);
 
 /*
+ * quest_hadamard_quantize_int4 with the rule for the scale as a parameter: QUEST_SCALE_GAUSSIAN is the reference's
+ * (benchmarks/utils.py:46, 207-208); QUEST_SCALE_ABSMAX sets scale = dtype(max|x| / 7.5 + 1e-8), the per-row absmax
+ * rule the CPU-runnable benchmark case names for its pre-quantised weights (no counterpart in the reference's code).
+ */
+#define QUEST_SCALE_GAUSSIAN 0
+#define QUEST_SCALE_ABSMAX 1
+int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
+                                      void *x_had, int group_size, int batch_size, float had_scale,
+                                      int scale_rule, int dtype, void *stream);
+
+/*
  * quest_hadamard_quantize_int4 with the producer of the activation in front, so that the normalised tensor is
  * never written: y = dtype(dtype(f32(x) * rsqrt(mean(x^2) + eps)) * norm_weight) -- the RMSNorm in front of every
  * attention and MLP block of the reference's model (src/models/llama.py:71-77, applied at llama.py:174-175) --

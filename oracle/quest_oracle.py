@@ -166,8 +166,20 @@ def fused_matmul_dequantize_int4_int4t(mat_a, mat_b, vec_a_add, vec_b_add, vec_a
 
 
 # ----------------------------------------------------------------------------- L1
-def preprocess_weight(weight: torch.Tensor, use_hadamard: bool = False):
-    """utils.py:20-49, dense branch.  Returns (w_int_packed, w_scale, w_add, None)."""
+def find_scale_absmax_int4(x: torch.Tensor, scale: torch.Tensor | None = None) -> torch.Tensor:
+    """The other weight-scale rule named for the CPU-runnable benchmark case ("per-row absmax scales"): the step
+    that puts the row's largest magnitude at the edge of the INT4 grid, 7.5 steps out (floor(x / s) is then 7 for
+    +absmax and -8 for -absmax, both dequantising to +-7.5 s).  Not in the reference's code, which uses the RMS
+    rule (utils.py:46); same epsilon as that rule so that an all-zero row is defined."""
+    if scale is None:
+        scale = torch.empty(*x.shape[:-1], 1, dtype=x.dtype)
+    scale_ = x.to(dtype=torch.float32).abs().amax(dim=-1, keepdim=True) / 7.5 + SCALE_EPS
+    return scale.copy_(scale_)
+
+
+def preprocess_weight(weight: torch.Tensor, use_hadamard: bool = False, w_scale_mode: str = 'rms'):
+    """utils.py:20-49, dense branch.  Returns (w_int_packed, w_scale, w_add, None).  w_scale_mode='rms' is the
+    reference's rule, 'absmax' the one above."""
     if use_hadamard:
         weight = hadamard128_fwht(weight, 2. ** -3.5)
     weight = weight.contiguous()
@@ -175,7 +187,7 @@ def preprocess_weight(weight: torch.Tensor, use_hadamard: bool = False):
     w_scale = torch.empty(n, 1, dtype=weight.dtype)
     w_int_packed = torch.empty(n, k // 2, dtype=torch.uint8)
     w_int_row_sum = torch.empty(n, 1, dtype=torch.int32)
-    find_scale_int4(weight, w_scale)
+    {'rms': find_scale_int4, 'absmax': find_scale_absmax_int4}[w_scale_mode](weight, w_scale)
     quantize_int4(weight, w_scale, None, w_int_packed.view(torch.int8), w_int_row_sum, False)
     w_add = w_int_row_sum + k // 2
     return w_int_packed, w_scale, w_add, None

@@ -171,12 +171,15 @@ def hadamard_quantize_int4(
         x_int_row_sum: torch.Tensor = None,
         x_had: torch.Tensor = None,
         hadamard_scale: float = HADAMARD_ENTRY,
+        scale_rule: str = 'gaussian',
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """One pass over x: block-128 Hadamard (skipped when hadamard_scale == 0), Gaussian-clip scale,
     INT4 codes packed two per byte, and their row sums -- the three launches of
     gemm-quest/benchmarks/utils.py:89-100 in one.  x_had, if given, receives the transformed
-    activations the codes were computed from.  Returns (scale, x_int_packed, x_int_row_sum)."""
+    activations the codes were computed from.  scale_rule: 'gaussian' (the reference's RMS rule) or 'absmax'
+    (scale = max|x| / 7.5 + 1e-8).  Returns (scale, x_int_packed, x_int_row_sum)."""
     m, k = x.shape
+    rule = {'gaussian': 0, 'absmax': 1}[scale_rule]
     if scale is None:
         scale = torch.empty(m, 1, dtype=x.dtype, device=x.device)
     if x_int_packed is None:
@@ -189,9 +192,9 @@ def hadamard_quantize_int4(
     assert x_had is None or (x_had.dtype == x.dtype and x_had.shape == x.shape and x_had.is_contiguous())
     dev = require_gpu(x, scale, x_int_packed, x_int_row_sum, x_had)
     with torch.cuda.device(dev):
-        check(_lib.load().quest_hadamard_quantize_int4(ptr(x), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum),
-                                                       ptr(x_had), k, m, float(hadamard_scale), DTYPE_CODE[x.dtype],
-                                                       stream_of(x)), 'hadamard_quantize_int4')
+        check(_lib.load().quest_hadamard_quantize_int4_rule(ptr(x), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum),
+                                                            ptr(x_had), k, m, float(hadamard_scale), rule,
+                                                            DTYPE_CODE[x.dtype], stream_of(x)), 'hadamard_quantize_int4')
     return scale, x_int_packed, x_int_row_sum
 
 

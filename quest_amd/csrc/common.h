@@ -144,6 +144,25 @@ __device__ __forceinline__ float block_sum_f(float v, float *slots) {
     __syncthreads();
     return t;
 }
+// The same for a maximum of non-negative values.
+template <int BLOCK>
+__device__ __forceinline__ float block_max_f(float v, float *slots) {
+    v = fmaxf(v, lane_xor_f<1>(v));
+    v = fmaxf(v, lane_xor_f<2>(v));
+    v = fmaxf(v, lane_xor_f<4>(v));
+    v = fmaxf(v, lane_xor_f<8>(v));
+    v = fmaxf(v, lane_xor_f<16>(v));
+    v = fmaxf(v, lane_xor_f<32>(v));
+    if constexpr (BLOCK == 64) return v;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    float t = slots[0];
+#pragma unroll
+    for (int w = 1; w < BLOCK / 64; w++) t = fmaxf(t, slots[w]);
+    __syncthreads();
+    return t;
+}
 template <int BLOCK>
 __device__ __forceinline__ int block_sum_i(int v, int *slots) {
     v = wave_sum_i(v);

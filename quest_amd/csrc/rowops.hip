@@ -85,7 +85,7 @@ template <int DT, int NCHUNK, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ scale,
                          uint32_t *__restrict__ packed, int32_t *__restrict__ row_sum,
-                         uint16_t *__restrict__ x_had, int K, float had_scale) {
+                         uint16_t *__restrict__ x_had, int K, float had_scale, int scale_rule) {
     __shared__ float slots_f[BLOCK / 64];
     __shared__ int slots_i[BLOCK / 64];
     const int row = blockIdx.x;
@@ -102,7 +102,7 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
     }
 
     float y[NCHUNK][8];
-    float sumsq = 0.f;
+    float sumsq = 0.f, amax = 0.f;
 #pragma unroll
     for (int i = 0; i < NCHUNK; i++) {
         unpack8<DT>(raw[i], y[i]);
@@ -114,7 +114,10 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
             unpack8<DT>(raw[i], y[i]);
         }
 #pragma unroll
-        for (int e = 0; e < 8; e++) sumsq += y[i][e] * y[i][e];     // squares of 16-bit floats are exact in fp32
+        for (int e = 0; e < 8; e++) {
+            sumsq += y[i][e] * y[i][e];         // squares of 16-bit floats are exact in fp32
+            amax = fmaxf(amax, fabsf(y[i][e]));
+        }
     }
     if (x_had != nullptr) {
         uint4 *hr = reinterpret_cast<uint4 *>(x_had + (size_t)row * K);
@@ -125,8 +128,16 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
         }
     }
 
-    const float total = block_sum_f<BLOCK>(sumsq, slots_f);
-    const uint32_t s16 = from_f32<DT>(scale_from_sumsq(total, K));
+    // QUEST_SCALE_GAUSSIAN: the reference's rule from the row's mean square; QUEST_SCALE_ABSMAX: the row's largest
+    // magnitude sits 7.5 steps out (a maximum is exact whatever the order, so this scale has no rounding slack)
+    uint32_t s16;
+    if (scale_rule == QUEST_SCALE_ABSMAX) {
+        const float m = block_max_f<BLOCK>(amax, slots_f);
+        s16 = from_f32<DT>(__fadd_rn(__fdiv_rn(m, 7.5f), kScaleEps));
+    } else {
+        const float total = block_sum_f<BLOCK>(sumsq, slots_f);
+        s16 = from_f32<DT>(scale_from_sumsq(total, K));
+    }
     if (tid == 0) scale[row] = (uint16_t)s16;
     const float s = to_f32<DT>(s16);
 
@@ -257,11 +268,11 @@ add_mul_vv_kernel(uint16_t *__restrict__ d, const int32_t *__restrict__ a_add, c
 // ---------------------------------------------------------------------------------------------
 template <int DT>
 static int launch_hadamard_quantize(const void *x, void *scale, uint8_t *packed, int32_t *row_sum, void *x_had,
-                                    int K, int M, float had_scale, hipStream_t st) {
+                                    int K, int M, float had_scale, int scale_rule, hipStream_t st) {
     const int nchunks = K >> 3;
 #define QUEST_HQ(NCH, BLK)                                                                              \
     hadamard_quantize_kernel<DT, NCH, BLK><<<dim3(M), dim3(BLK), 0, st>>>(                              \
-        (const uint16_t *)x, (uint16_t *)scale, (uint32_t *)packed, row_sum, (uint16_t *)x_had, K, had_scale)
+        (const uint16_t *)x, (uint16_t *)scale, (uint32_t *)packed, row_sum, (uint16_t *)x_had, K, had_scale, scale_rule)
     if (nchunks <= 256) QUEST_HQ(1, 256);
     else if (nchunks <= 512) QUEST_HQ(2, 256);
     else if (nchunks <= 1024) QUEST_HQ(4, 256);
@@ -387,8 +398,29 @@ extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t 
                                                  group_size, batch_size, had_scale, dtype, st);
     if (rc != QUEST_ERR_UNSUPPORTED) return rc;
     if (dtype == QUEST_DTYPE_BF16)
-        return launch_hadamard_quantize<0>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale, st);
-    return launch_hadamard_quantize<1>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale, st);
+        return launch_hadamard_quantize<0>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale,
+                                           QUEST_SCALE_GAUSSIAN, st);
+    return launch_hadamard_quantize<1>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale,
+                                       QUEST_SCALE_GAUSSIAN, st);
+}
+
+extern "C" int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
+                                                 void *x_had, int group_size, int batch_size, float had_scale,
+                                                 int scale_rule, int dtype, void *stream) {
+    if (scale_rule == QUEST_SCALE_GAUSSIAN)
+        return quest_hadamard_quantize_int4(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale,
+                                            dtype, stream);
+    if (scale_rule != QUEST_SCALE_ABSMAX) return QUEST_ERR_BAD_SHAPE;
+    if (!x || !scale) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(x, 16) || !aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == QUEST_DTYPE_BF16)
+        return launch_hadamard_quantize<0>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale,
+                                           scale_rule, st);
+    return launch_hadamard_quantize<1>(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale,
+                                       scale_rule, st);
 }
 
 extern "C" int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *norm_weight, float eps, void *scale,

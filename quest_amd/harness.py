@@ -82,7 +82,8 @@ def fused_matmul_dequantize_int4_bf16(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_
     return mat_d
 
 
-def preprocess_weight(weight: torch.Tensor, use_sparse: bool = False, use_hadamard: bool = False, backend: str = 'hip'):
+def preprocess_weight(weight: torch.Tensor, use_sparse: bool = False, use_hadamard: bool = False, backend: str = 'hip',
+                      w_scale_mode: str = 'rms'):
     """utils.py:20-53, dense branch: (N, K) float weight -> (w_int_packed (N, K/2) uint8,
     w_scale (N, 1), w_add (N, 1) int32 = row sum of the codes + K/2, None)."""
     _check_backend(backend)
@@ -94,8 +95,10 @@ def preprocess_weight(weight: torch.Tensor, use_sparse: bool = False, use_hadama
     w_int_packed = torch.empty(n, k // 2, dtype=torch.uint8, device=weight.device)
     w_int_row_sum = torch.empty(n, 1, dtype=torch.int32, device=weight.device)
     # one pass: weight-side Hadamard (scale 2^-3.5) when asked, then scale, codes and row sums
+    # (w_scale_mode: 'rms' is the reference's rule, 'absmax' puts the row's largest magnitude at the grid's edge)
     quest.hadamard_quantize_int4(weight, w_scale, w_int_packed, w_int_row_sum,
-                                 hadamard_scale=WEIGHT_HADAMARD_SCALE if use_hadamard else 0.)
+                                 hadamard_scale=WEIGHT_HADAMARD_SCALE if use_hadamard else 0.,
+                                 scale_rule={'rms': 'gaussian', 'absmax': 'absmax'}[w_scale_mode])
     w_add = w_int_row_sum + k // 2
     return w_int_packed, w_scale, w_add, None
 

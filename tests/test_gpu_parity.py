@@ -266,6 +266,24 @@ def test_hadamard_quantize_weight_scale_runs_butterflies(quest, dtype):
     assert torch.equal(packed.cpu(), xp) and torch.equal(row_sum.cpu(), rs)
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('use_hadamard', [False, True])
+def test_preprocess_weight_absmax_bit_exact(quest, dtype, use_hadamard):
+    """The absmax scale rule: a maximum has no summation order, so scale, codes and sums all match bit for bit."""
+    from quest_amd import harness
+    w = (torch.randn(200, 1152, generator=torch.Generator().manual_seed(14)) * 0.02).to(dtype)
+    wp, ws, wa, _ = harness.preprocess_weight(w.to(DEV), use_hadamard=use_hadamard, w_scale_mode='absmax')
+    op, os_, oa, _ = qo.preprocess_weight(w, use_hadamard=use_hadamard, w_scale_mode='absmax')
+    assert torch.equal(bits(ws.cpu()), bits(os_))
+    assert torch.equal(wp.cpu(), op) and torch.equal(wa.cpu(), oa)
+    # and the reference's rule through the same entry point is unchanged
+    wp2, ws2, wa2, _ = harness.preprocess_weight(w.to(DEV), use_hadamard=use_hadamard)
+    op2, os2, oa2, _ = qo.preprocess_weight(w, use_hadamard=use_hadamard)
+    assert ulp_diff(ws2, os2).max() <= 1
+    if torch.equal(bits(ws2.cpu()), bits(os2)):
+        assert torch.equal(wp2.cpu(), op2) and torch.equal(wa2.cpu(), oa2)
+
+
 # --------------------------------------------------------------------------- producers fused in front
 def _ulp_stats(got, want):
     d = ulp_diff(got, want)

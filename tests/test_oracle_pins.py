@@ -357,3 +357,35 @@ def test_linear_forward_hadamard_rotation_preserves_product():
     a = qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='matmul')
     b = qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='fwht')
     assert ((a.double() - b.double()).norm() / a.double().norm()) < 1e-2
+
+
+# --------------------------------------------------------------------------- the absmax weight-scale rule
+def test_absmax_scale_closed_forms():
+    """Row maximum 7.5 -> step exactly 1 (+1e-8 vanishes in 16 bits): +7.5 gets code 7, -7.5 code -8, both
+    dequantise to +-7.5; a zero row gets the epsilon alone."""
+    for dtype in (torch.bfloat16, torch.float16):
+        x = torch.tensor([[7.5, -7.5, 0.4, -0.4, 3.0, 0.0, 6.5, -1.0]], dtype=dtype)
+        s = qo.find_scale_absmax_int4(x)
+        assert float(s) == 1.0
+        q = torch.empty(1, 8, dtype=torch.int8)
+        qo.quantize_int4(x.clone(), s, q, None, None, False)
+        assert q.tolist() == [[7, -8, 0, -1, 3, 0, 6, -1]]
+        z = qo.find_scale_absmax_int4(torch.zeros(2, 128, dtype=dtype))
+        assert torch.equal(z, torch.full((2, 1), 1e-8).to(dtype))
+    x = torch.randn(64, 256, generator=torch.Generator().manual_seed(3)).bfloat16()
+    s = qo.find_scale_absmax_int4(x).float()
+    amax = x.float().abs().amax(-1, keepdim=True)
+    assert ((s - amax / 7.5).abs() <= amax / 7.5 * 2. ** -8).all()
+
+
+def test_preprocess_weight_absmax_never_clips_beyond_the_grid():
+    w = (torch.randn(32, 256, generator=torch.Generator().manual_seed(4)) * 0.02).bfloat16()
+    for had in (False, True):
+        packed, scale, add, _ = qo.preprocess_weight(w, use_hadamard=had, w_scale_mode='absmax')
+        codes = qo.unpack_int4(packed)
+        assert codes.min() >= -8 and codes.max() <= 7
+        assert torch.equal(add, codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + 128)
+        wt = qo.hadamard128_fwht(w, 2. ** -3.5) if had else w
+        deq = (codes.float() + .5) * scale.float()
+        # inside the grid the error is at most half a step (plus the rounding of the scale itself)
+        assert ((deq - wt.float()).abs() <= scale.float() * 0.51).all()
