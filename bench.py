@@ -269,7 +269,7 @@ def bench_cpu_baseline():
     m, k, n = 512, 1024, 1024
     x = torch.randn(m, k).half()
     w = (torch.randn(n, k) * 0.02).half()
-    wp, ws, wa, _ = qo.preprocess_weight(w, use_hadamard=True)
+    wp, ws, wa, _ = qo.preprocess_weight(w, use_hadamard=True, w_scale_mode='absmax')      # pre-quantised, per-row absmax scales
     for _ in range(3):
         qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='matmul', via='fp64')
     times = []

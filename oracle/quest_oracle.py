@@ -230,3 +230,31 @@ def linear_fp64(a_int, a_scale, w_int, w_scale):
     a_dq = (a_int.to(torch.float64) + .5) * a_scale.to(torch.float64)
     w_dq = (w_int.to(torch.float64) + .5) * w_scale.to(torch.float64)
     return a_dq @ w_dq.t()
+
+
+# ---------------------------------------------------------------------------------------------
+# The training-side (fake-quantised) statement of the same layer, for judging the packed INT4 path
+# against what a QuEST-trained checkpoint was evaluated with.
+# ---------------------------------------------------------------------------------------------
+OPTIMAL_GAUSSIAN_SCALE_INT4 = 2.513930578568423      # src/models/quantization/base_linear.py:38-48, bits = 4
+
+
+def fake_quant_hadamard(x: torch.Tensor):
+    """src/eval_hswag.py:203-217 (quantize_pack_hadamard_dense, 4 bits, centred): rotate by the block-128 Hadamard
+    transform (factor 2^-3.5), clip at 2.5139 rms, round to the 16 levels.  Returns (levels 0..15 in the rotated
+    space, scale, step), all fp32."""
+    xf = x.to(torch.float32)
+    x_had = hadamard128_fwht(xf.reshape(-1, HADAMARD_BLOCK), 2. ** -3.5, out_dtype=torch.float32).reshape(x.shape)
+    std = torch.sqrt(torch.mean(x_had ** 2, dim=-1, keepdim=True)) + 1e-8
+    scale = OPTIMAL_GAUSSIAN_SCALE_INT4 * std
+    step = 2 * scale / 15
+    xq = torch.round((torch.clamp(x_had, -scale, scale) + scale) / step)
+    return xq, scale, step
+
+
+def fake_quant_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """src/eval_hswag.py:156-173 (its Linear4bit): both operands fake-quantised in the rotated space, dense fp32
+    product.  The rotations cancel in the product, so this is the layer the packed path computes."""
+    xq, xs, xstep = fake_quant_hadamard(x)
+    wq, ws, wstep = fake_quant_hadamard(weight)
+    return F.linear(xq * xstep - xs, wq * wstep - ws, None if bias is None else bias.to(torch.float32))

@@ -259,6 +259,31 @@ def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, 
     return model
 
 
+@torch.no_grad()
+def load_reference_state_dict(model: Llama, state_dict: dict) -> Llama:
+    """Copy the weights of a checkpoint of the reference's model (src/models/llama.py; parameter names
+    `transformer.wte.weight`, `transformer.h.<i>.attn.c_attn.weight`, ..., `lm_head.weight`, possibly behind the
+    `_orig_mod.module.` prefix its training wrapper adds, src/eval_hswag.py:187-195) into a dense model of this
+    module; quantiser buffers and other non-parameter entries are ignored.  `quantize_model` then packs the linears:
+    the weight quantiser the reference trains with (Hadamard, Gaussian clip, 16 levels) is the grid
+    `preprocess_weight(use_hadamard=True)` produces, so the trained weights map to INT4 codes directly."""
+    own = model.state_dict()
+    picked = {}
+    for name, value in state_dict.items():
+        for prefix in ('_orig_mod.module.', 'module.', ''):
+            if name.startswith(prefix) and name[len(prefix):] in own:
+                picked[name[len(prefix):]] = value
+                break
+    missing = [k for k in own if k not in picked]
+    if missing:
+        raise KeyError(f'checkpoint lacks {len(missing)} parameters, e.g. {missing[:3]}')
+    for k, v in picked.items():
+        if own[k].shape != v.shape:
+            raise ValueError(f'{k}: checkpoint shape {tuple(v.shape)} != model shape {tuple(own[k].shape)}')
+        own[k].copy_(v)
+    return model
+
+
 @torch.inference_mode()
 def bench_forward(model: Llama, batch_size: int, seq_len: int, n_warmup: int = 5, n_iter: int = 10) -> dict:
     """bench_e2e.py:99-121: seconds per forward, eagerly and as a replayed HIP graph (the smaller is the

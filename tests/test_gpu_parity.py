@@ -284,6 +284,28 @@ def test_preprocess_weight_absmax_bit_exact(quest, dtype, use_hadamard):
         assert torch.equal(wp2.cpu(), op2) and torch.equal(wa2.cpu(), oa2)
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_packed_linear_against_training_side_fake_quant(quest, dtype):
+    """The layer a QuEST-trained checkpoint was evaluated with (fake quantisation in fp32, src/eval_hswag.py of the
+    reference) against the packed INT4 layer built from the same dense weight.  The inference path rounds the rotated
+    activations to 16 bits before quantising (benchmarks/utils.py:89-90), which moves a per cent or two of the codes
+    to the neighbouring level: measured 3.4e-2 relative in bf16 and 1.2e-2 in fp16, for this kernel and for the
+    CPU oracle of the reference's inference path alike -- the distance belongs to the path, not to the kernel."""
+    from quest_amd import harness
+    g = torch.Generator().manual_seed(40)
+    x = torch.randn(192, 1024, generator=g).to(dtype)
+    w = (torch.randn(320, 1024, generator=g) * 0.02).to(dtype)
+    want = qo.fake_quant_linear(x, w).double()
+    layer = harness.Linear4bit.from_weight(w.to(DEV), use_hadamard=True)
+    got = layer(x.to(DEV)).double().cpu()
+    wp, ws, wa, _ = qo.preprocess_weight(w, use_hadamard=True)
+    ref = qo.linear_forward(x, wp, ws, wa, use_hadamard=True, hadamard='matmul', via='fp32').double()
+    err = (got - want).norm() / want.norm()
+    err_ref = (ref - want).norm() / want.norm()
+    assert err < (5e-2 if dtype == torch.bfloat16 else 2e-2), float(err)
+    assert err < 1.25 * err_ref + 1e-3, (float(err), float(err_ref))
+
+
 # --------------------------------------------------------------------------- producers fused in front
 def _ulp_stats(got, want):
     d = ulp_diff(got, want)

@@ -132,3 +132,16 @@ def test_load_rejects_other_files(tmp_path):
     save_file({'a': torch.zeros(2)}, path, metadata={'format': 'something-else'})
     with pytest.raises(ValueError):
         checkpoint.read_metadata(path)
+
+
+def test_reference_checkpoint_names_load():
+    model, cfg = tiny_model()
+    src, _ = tiny_model(seed=9)
+    sd = {'_orig_mod.module.' + k: v for k, v in src.state_dict().items()}
+    sd['_orig_mod.module.transformer.h.0.attn.c_attn.weight_quantizer.some_buffer'] = torch.zeros(1)
+    llama.load_reference_state_dict(model, sd)
+    for (ka, va), (kb, vb) in zip(model.state_dict().items(), src.state_dict().items()):
+        assert ka == kb and torch.equal(va, vb)
+    del sd['_orig_mod.module.lm_head.weight']
+    with pytest.raises(KeyError):
+        llama.load_reference_state_dict(model, sd)

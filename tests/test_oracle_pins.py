@@ -389,3 +389,37 @@ def test_preprocess_weight_absmax_never_clips_beyond_the_grid():
         deq = (codes.float() + .5) * scale.float()
         # inside the grid the error is at most half a step (plus the rounding of the scale itself)
         assert ((deq - wt.float()).abs() <= scale.float() * 0.51).all()
+
+
+# --------------------------------------------------------------------------- training-side fake quantisation
+def test_fake_quant_grid_is_the_inference_grid():
+    """The 16 levels of the training-side quantiser, (k - 7.5) step for k = 0..15, are the inference grid
+    (q + 1/2) s with q = k - 8 and s = step; round-to-level and floor-to-code pick the same level except at exact
+    ties and where the two scale formulas (epsilon inside or outside the product) differ in the last bits."""
+    x = torch.randn(64, 512, generator=torch.Generator().manual_seed(11))
+    xq, scale, step = qo.fake_quant_hadamard(x)
+    assert xq.min() >= 0 and xq.max() <= 15
+    deq = xq * step - scale
+    assert torch.allclose(deq, (xq - 7.5) * step, atol=1e-6)
+    x_had = qo.hadamard128_fwht(x, 2. ** -3.5)
+    s = qo.find_scale_int4(x_had)
+    assert torch.allclose(s, step, rtol=1e-6)
+    codes = torch.empty(64, 512, dtype=torch.int8)
+    qo.quantize_int4(x_had.clone(), s, codes, None, None, False)
+    assert ((codes.float() + 8) != xq).float().mean() < 1e-3
+
+
+def test_fake_quant_linear_equals_packed_linear_in_exact_arithmetic():
+    """fp32 end to end on both sides (no 16-bit rounding anywhere): the packed path's integer GEMM and scale
+    epilogue reproduce the fake-quantised dense product up to the handful of codes on a rounding tie."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(32, 256, generator=g)
+    w = torch.randn(48, 256, generator=g) * 0.02
+    want = qo.fake_quant_linear(x, w)
+    xq, xs, xstep = qo.fake_quant_hadamard(x)
+    wq, ws, wstep = qo.fake_quant_hadamard(w)
+    a, b = (xq - 8).to(torch.int64), (wq - 8).to(torch.int64)
+    c = a @ b.t()
+    lhs = (2 * c + a.sum(-1, keepdim=True) + (b.sum(-1, keepdim=True) + 128).t()).double()
+    got = lhs * (0.5 * xstep.double() * wstep.double().t())
+    assert torch.allclose(got, want.double(), rtol=1e-4, atol=1e-6)
