@@ -145,6 +145,9 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
     v4u bq[8];
 #pragma unroll
     for (int s = 0; s < 8; s++) bq[s] = __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(ld_off + 32 * s), 0, 0);
+    // all eight in flight before anything else: left alone the scheduler sinks the last two below the first MFMAs to
+    // save registers, which costs every wave a second trip to memory
+    __builtin_amdgcn_sched_barrier(0);
 
     if constexpr (PRE == kPreRmsNorm) {
         const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, 0x00020000);
