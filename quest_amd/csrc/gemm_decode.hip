@@ -100,6 +100,9 @@ gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
                     aq[i][t][hlf] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, (int)(in_row ? a_off[t] + shift : dead), 0, 0));
             }
         }
+        // every load of the batch in flight before the first is used (the scheduler would otherwise sink some of
+        // them between the MFMAs to save registers and pay a second trip to memory)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < kBatch; i++)
 #pragma unroll
