@@ -33,14 +33,15 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 REPLAYS = 7                  # timed replays of a batch of launches; the median is reported
+EAGER_BATCHES = False        # --eager-batches: time plain launches instead of graph replays
 LAST = {'min_ms': None}      # fastest replay of the most recent launches_ms() call
 INT8_MFMA_PEAK_TOPS = 5000.0
 
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
 # scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.99980, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
-TRAFFIC_GEMM_BYTES = 358800835          # M=4096 K=4096 N=11008 fp16: (118931.1 x 1.99980 + 112553.2) KiB
-TRAFFIC_QUANTIZE_BYTES = 84105907       # bf16 [8192, 4096]: (32814.2 x 1.99980 + 16512.9) KiB
+TRAFFIC_GEMM_BYTES = 359763152
+TRAFFIC_QUANTIZE_BYTES = 84095204
 
 
 def event_pairs(n):
@@ -64,6 +65,19 @@ def launches_ms(launch, n, warmup=5):
     for i in range(warmup):
         launch(i)
     torch.cuda.synchronize()
+    if EAGER_BATCHES:                            # plain launches (counter collection cannot follow graph replays)
+        per_launch = []
+        for _ in range(REPLAYS):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for i in range(n):
+                launch(i)
+            b.record()
+            torch.cuda.synchronize()
+            per_launch.append(a.elapsed_time(b) / n)
+        per_launch.sort()
+        LAST['min_ms'] = per_launch[0]
+        return per_launch[len(per_launch) // 2]
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -127,13 +141,18 @@ def bench_linear(quest, _lib, steps, warmup, dev):
 
     for i in range(warmup):
         step(i)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        step(i, evs[i])
+        step(i)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    # the split between the two kernels, from a second pass with events between them (the events cost a few
+    # microseconds each, which is why the timed pass above has none)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for i in range(steps):
+        step(i, evs[i])
+    torch.cuda.synchronize()
     quant_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
     gemm_in_step_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
 
@@ -346,7 +365,11 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-forward', action='store_true', help='skip the whole-model row')
+    ap.add_argument('--eager-batches', action='store_true',
+                    help='time batches of plain launches instead of HIP-graph replays (for rocprofv3 --pmc runs)')
     args = ap.parse_args()
+    global EAGER_BATCHES
+    EAGER_BATCHES = args.eager_batches
     if args.gpus != 1:
         sys.exit('bench.py: this build runs on one GPU; --gpus above 1 is not supported '
                  '(the path shards by tokens with no exchange, but no multi-GPU run is part of it)')

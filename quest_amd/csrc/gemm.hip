@@ -532,6 +532,9 @@ __device__ __forceinline__ void cursor_next_tile(Cursor &c) {
     if (c.left <= 0) { c.valid = false; return; }             // keeps pointing at the last tile
     int width = c.nug - c.u;
     width = width < c.left ? width : c.left;
+    // kept in a scalar register: two chained minima would otherwise be selected as the vector ALU's three-operand
+    // minimum, which drags the whole cursor into vector registers (and those get spilled at the register peaks)
+    asm volatile("" : "+s"(width));
     width = width < kMaxUnits ? width : kMaxUnits;
     c.tok0 = c.tt * kRows;
     c.ch0 = (c.ug0 + c.u) * 32;
@@ -541,6 +544,13 @@ __device__ __forceinline__ void cursor_next_tile(Cursor &c) {
     c.left -= width;
     c.u += width;
     if (c.u == c.nug) { c.u = 0; c.tt++; }
+}
+
+// lane number from the execution mask (volatile: never merged with an earlier copy)
+__device__ __forceinline__ int fresh_lane_id() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
 }
 
 struct Loader {          // direct-to-LDS loads of one wave: 4 instructions of 16 token rows, 4 of 16 channel rows
@@ -575,17 +585,17 @@ __device__ __forceinline__ void loader_one(const Loader &l, const Cursor &ld, ui
         __builtin_amdgcn_raw_ptr_buffer_load_lds(l.wgt, (__attribute__((address_space(3))) void *)(sb + kTileB + (j - 4) * 16 * kRowB),
                                                  16, l.off_c, kb + (j - 4) * step, 0, 0);
 }
-__device__ __forceinline__ void loader_end(Loader &l, Cursor &ld, int lane) {
+__device__ __forceinline__ void loader_end(Loader &l, Cursor &ld) {
     l.issued++;
     if (++ld.kt == l.nk) {
         cursor_next_tile(ld);
-        if (ld.valid) loader_offsets(l, ld, lane); else ld.kt = l.nk - 1;
+        if (ld.valid) loader_offsets(l, ld, fresh_lane_id()); else ld.kt = l.nk - 1;
     }
 }
-__device__ __forceinline__ void loader_issue(Loader &l, Cursor &ld, uint8_t *lds, int lane) {
+__device__ __forceinline__ void loader_issue(Loader &l, Cursor &ld, uint8_t *lds) {
 #pragma unroll
     for (int j = 0; j < kLoads; j++) loader_one(l, ld, lds, j);
-    loader_end(l, ld, lane);
+    loader_end(l, ld);
 }
 
 template <int N>
@@ -603,13 +613,6 @@ __device__ __forceinline__ void wait_stage(int extra) {
         case 4: wait_vmcnt_imm<kBase + 4>(); break;
         default: wait_vmcnt_imm<kBase>(); break;
     }
-}
-
-// lane number from the execution mask (volatile: never merged with an earlier copy)
-__device__ __forceinline__ int fresh_lane_id() {
-    int l;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
-    return l;
 }
 
 struct Pipe {            // state that lives across tiles
@@ -690,9 +693,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                                          int unit0, int width) {
     constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
     constexpr int NAX = NA > 0 ? NA : 1;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps everything derived from it in scalar registers
+    // Lane coordinates are derived afresh in every phase (here, in the loader's cursor step, in the epilogue): a value
+    // computed once from threadIdx would be kept alive across the whole kernel, spilled to scratch at the register
+    // peaks, and a scratch reload waits on the vector-memory counter, i.e. on every store and load in flight.
+    const int lane = fresh_lane_id();
+    const int wave = ldr.wave;                                      // scalar
     const int wt = wave >> 1;
     const int li = lane & 31;
     const int lg = lane >> 5;
@@ -747,10 +752,10 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         if (pp.store_syncs > 0) { wait_stage(pp.store_extra); pp.store_syncs--; } else { wait_stage(0); }
         plain_barrier();
     };
-    auto dma = [&](int j) { if (j < kLoads) loader_one(ldr, ld, lds, j); else loader_end(ldr, ld, lane); };
+    auto dma = [&](int j) { if (j < kLoads) loader_one(ldr, ld, lds, j); else loader_end(ldr, ld); };
     auto no_sync = []() {};
     if constexpr (NA == 0) {
-        for (int kt = 0; kt < nk; kt++) { sync(); loader_issue(ldr, ld, lds, lane); pp.it++; }
+        for (int kt = 0; kt < nk; kt++) { sync(); loader_issue(ldr, ld, lds); pp.it++; }
     } else {
         Frags u0, u1;
         {   // prologue: the first k-pair of the tile's first stage (landed: the previous synchronisation saw to it)
@@ -915,28 +920,30 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
                      const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
                      int M, int N, int K, stream::Schedule sch) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsB];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
     // wave-uniform by construction; readfirstlane tells the compiler so, which keeps everything that is
-    // updated under `switch (na)` below (cursors, slot numbers, LDS bases) in scalar registers
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // updated under `switch (na)` below (cursors, slot numbers, LDS bases) in scalar registers; the empty
+    // asm cuts the value loose from threadIdx, which would otherwise be kept (and spilled) to derive it again
+    int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    asm volatile("" : "+s"(wave));
     const int wc = wave & 1;                     // channel half this wave multiplies
     const int kbytes = K >> 1;
 
-    const int grp = blockIdx.x % sch.groups;
-    const int rank = blockIdx.x / sch.groups;
-    const int per_grp = gridDim.x / sch.groups;
-    const int ug0 = (int)(((long)grp * sch.units) / sch.groups);
-    const int ug1 = (int)(((long)(grp + 1) * sch.units) / sch.groups);
+    const int rank = __builtin_amdgcn_readfirstlane((int)(blockIdx.x / sch.groups));
+    const int grp = blockIdx.x - rank * sch.groups;
+    const int per_grp = __builtin_amdgcn_readfirstlane((int)(gridDim.x / sch.groups));
+    const int ug0 = __builtin_amdgcn_readfirstlane((int)(((long)grp * sch.units) / sch.groups));
+    const int ug1 = __builtin_amdgcn_readfirstlane((int)(((long)(grp + 1) * sch.units) / sch.groups));
     Cursor cc, ld;
     cc.nug = ug1 - ug0;
     cc.ug0 = ug0;
+    // the divisions run on the vector ALU (there is no scalar divide); readfirstlane brings the (uniform) results
+    // back to scalar registers, and with them the whole cursor arithmetic of the tile loop
     const long cells = (long)sch.tiles_t * cc.nug;
-    const long pos0 = (cells * rank) / per_grp;
-    const long pos1 = (cells * (rank + 1)) / per_grp;
-    cc.tt = (int)(pos0 / cc.nug);
-    cc.u = (int)(pos0 % cc.nug);
-    cc.left = (int)(pos1 - pos0);
+    const int pos0 = __builtin_amdgcn_readfirstlane((int)((cells * rank) / per_grp));
+    const int pos1 = __builtin_amdgcn_readfirstlane((int)((cells * (rank + 1)) / per_grp));
+    cc.tt = __builtin_amdgcn_readfirstlane(pos0 / cc.nug);
+    cc.u = pos0 - cc.tt * cc.nug;
+    cc.left = pos1 - pos0;
     cc.valid = false;
     cc.tok0 = cc.ch0 = cc.width = cc.kt = 0;
     ld = cc;
@@ -955,11 +962,11 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     ldr.nk = K / 128;
     ldr.wave = wave;
     ldr.issued = 0;
-    loader_offsets(ldr, ld, lane);
+    loader_offsets(ldr, ld, fresh_lane_id());
 
     // ---- pipeline prologue: stages 0 .. kStages - 2 in flight, stage 0 landed
 #pragma unroll
-    for (int s = 0; s < kStages - 1; s++) loader_issue(ldr, ld, lds, lane);
+    for (int s = 0; s < kStages - 1; s++) loader_issue(ldr, ld, lds);
     wait_vmcnt_imm<kLoads * (kStages - 2)>();
     plain_barrier();
     Pipe pp;
