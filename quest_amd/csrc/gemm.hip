@@ -487,29 +487,43 @@ gemm_w4a4_stream_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
 // =================================================================================================
 // Large-tile persistent kernel (K % 128 == 0): the prefill path
 // =================================================================================================
-// One workgroup of four waves per CU owns 256 tokens x up to 256 channels; wave w multiplies tokens
+// A workgroup of four waves owns 256 tokens x up to 256 (or 128) channels; wave w multiplies tokens
 // [128 (w >> 1), +128) by the lower or upper half of the tile's channel units (up to 128 x 128 per
 // wave: 4 x 4 accumulators in the AGPR half of the 512 registers a lone wave per SIMD has).
-// Compared with the 128-channel kernel above this halves the L2 -> CU bytes per multiply, and
-// compared with staging int8 through registers it keeps the LDS pipe (the measured bottleneck of
+// Compared with staging int8 through registers this keeps the LDS pipe (the measured bottleneck of
 // that variant) at a third of the traffic: packed bytes go HBM -> LDS directly
-// (buffer_load_dwordx4 ... lds, four stages of 32 KiB), a lane reads 16 packed bytes of one row
+// (buffer_load_dwordx4 ... lds, stages of 128 k), a lane reads 16 packed bytes of one row
 // and splits them into the int8 vectors of 16 * (even-k nibbles) and 16 * (odd-k nibbles), which
 // feed two MFMA k-steps.  The stage pipeline runs on across the workgroup's tiles, and the
 // epilogue's stores are left to drain under the next tile's first stages.
 namespace big {
 
-constexpr int kRows = 256;                    // rows of either operand per tile
-constexpr int kMaxUnits = 8;                  // channel units (32 rows) per tile
+constexpr int kRows = 256;                    // token rows per tile
 constexpr int kRowB = 64;                     // packed bytes per row per stage (128 k)
-constexpr int kTileB = kRows * kRowB;         // 16 KiB
-constexpr int kStageB = 2 * kTileB;           // token tile + channel tile
-constexpr int kStages = 4;
-constexpr int kLoads = 8;                     // buffer loads per wave per stage
-constexpr int kVecOff = kStages * kStageB;
+constexpr int kTileB = kRows * kRowB;         // 16 KiB: the token rows of a stage; the channel rows follow
 constexpr int kVecParB = 2 * (kRows * 4 + kRows * 2);   // b_add, b_mul per channel and a_add, a_mul per token of one tile
 constexpr int kVecB = 2 * kVecParB;                       // two tiles in flight
-constexpr int kLdsB = kVecOff + kVecB;        // 134 KiB of the CU's 160 KiB
+
+// Two shapes of the same kernel:
+//   Wide: 256 x 256 tiles, one workgroup per CU, a wave holds 128 x 128 (256 accumulator registers) and both
+//         fragment sets of the software pipeline; nothing else runs on its SIMD, so the epilogue idles the matrix pipe.
+//   Duo:  256 x 128 tiles, two workgroups per CU, a wave holds 128 x 64; the two waves of a SIMD belong to different
+//         tiles, so one tile's epilogue and synchronisation waits run under the other's multiplications.  Costs 1.5 x
+//         the operand traffic and nibble splitting per multiply; wins where the wide shape's tiles would be narrow
+//         or few (few channels) and where K is short, i.e. where the epilogue weighs most.
+template <int MAXU, int STAGES, int WGS>
+struct Cfg {
+    static constexpr int kMaxUnits = MAXU;                    // channel units (32 rows) per tile
+    static constexpr int kChnRowsPerWave = 8 * MAXU;          // channel rows each wave loads per stage
+    static constexpr int kStageB = kTileB + 32 * MAXU * kRowB;
+    static constexpr int kStages = STAGES;
+    static constexpr int kLoads = 4 + MAXU / 2;               // buffer loads per wave per stage (16 rows each)
+    static constexpr int kVecOff = STAGES * kStageB;
+    static constexpr int kLdsB = kVecOff + kVecB;             // Wide: 134 KiB, Duo: 78 KiB of the CU's 160 KiB
+    static constexpr int kWgPerCu = WGS;
+};
+using Wide = Cfg<8, 4, 1>;
+using Duo = Cfg<4, 3, 2>;
 
 // s_barrier alone: waves order their own LDS traffic with s_waitcnt, and a release / acquire fence here would
 // make the compiler drain every direct-to-LDS load still in flight (vmcnt(0)), which is the pipeline
@@ -528,6 +542,7 @@ struct Cursor {          // walks a workgroup's run of cells tile by tile, stage
     bool valid;
 };
 
+template <typename C>
 __device__ __forceinline__ void cursor_next_tile(Cursor &c) {
     if (c.left <= 0) { c.valid = false; return; }             // keeps pointing at the last tile
     int width = c.nug - c.u;
@@ -535,7 +550,7 @@ __device__ __forceinline__ void cursor_next_tile(Cursor &c) {
     // kept in a scalar register: two chained minima would otherwise be selected as the vector ALU's three-operand
     // minimum, which drags the whole cursor into vector registers (and those get spilled at the register peaks)
     asm volatile("" : "+s"(width));
-    width = width < kMaxUnits ? width : kMaxUnits;
+    width = width < C::kMaxUnits ? width : C::kMaxUnits;
     c.tok0 = c.tt * kRows;
     c.ch0 = (c.ug0 + c.u) * 32;
     c.width = width;
@@ -553,49 +568,54 @@ __device__ __forceinline__ int fresh_lane_id() {
     return l;
 }
 
-struct Loader {          // direct-to-LDS loads of one wave: 4 instructions of 16 token rows, 4 of 16 channel rows
+struct Loader {          // direct-to-LDS loads of one wave: 4 instructions of 16 token rows, 2 or 4 of 16 channel rows
     __amdgpu_buffer_rsrc_t act, wgt, badd, bmul, aadd, amul;
     uint32_t off_t, off_c;      // byte offset of this lane's first row of the load cursor's tile (+ its 16-byte chunk)
     int kbytes, nk, wave;
     int issued;                 // stages issued so far by this workgroup (slot = issued % kStages)
 };
 
+template <typename C>
 __device__ __forceinline__ void loader_offsets(Loader &l, const Cursor &ld, int lane) {
     // lane p of an instruction covers row p / 4 of its 16 rows; LDS slot p (lane order) must hold chunk
     // (p & 3) ^ ((row >> 2) & 3) of that row, so the lane fetches exactly that chunk
-    const int row = l.wave * 64 + (lane >> 2);
+    const int row = lane >> 2;
     const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
-    l.off_t = (uint32_t)(ld.tok0 + row) * (uint32_t)l.kbytes + chunk * 16;
-    l.off_c = (uint32_t)(ld.ch0 + row) * (uint32_t)l.kbytes + chunk * 16;
+    l.off_t = (uint32_t)(ld.tok0 + l.wave * 64 + row) * (uint32_t)l.kbytes + chunk * 16;
+    l.off_c = (uint32_t)(ld.ch0 + l.wave * C::kChnRowsPerWave + row) * (uint32_t)l.kbytes + chunk * 16;
 }
 
-// The load cursor's stage goes into the next LDS slot as eight instructions per wave (loader_one, j = 0..7: four of
-// 16 token rows, four of 16 channel rows), issued a few MFMAs apart because each takes the CU's address path about
+// The load cursor's stage goes into the next LDS slot as kLoads instructions per wave (loader_one: four of
+// 16 token rows, then those of 16 channel rows), issued a few MFMAs apart because each takes the CU's address path about
 // half an MFMA; loader_end then advances the cursor (into the next tile when this one is done; when nothing is
 // left the last stage is fetched again, which keeps the count of outstanding loads uniform).
 // Rows past the end of a matrix read as zeros.
+template <typename C>
 __device__ __forceinline__ void loader_one(const Loader &l, const Cursor &ld, uint8_t *lds, int j) {
-    uint8_t *sb = lds + (l.issued % kStages) * kStageB + l.wave * 64 * kRowB;
+    uint8_t *sb = lds + (l.issued % C::kStages) * C::kStageB;
     const int kb = ld.kt * kRowB;
     const int step = 16 * l.kbytes;
     if (j < 4)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.act, (__attribute__((address_space(3))) void *)(sb + j * 16 * kRowB), 16,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.act, (__attribute__((address_space(3))) void *)(sb + (l.wave * 64 + j * 16) * kRowB), 16,
                                                  l.off_t, kb + j * step, 0, 0);
     else
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(l.wgt, (__attribute__((address_space(3))) void *)(sb + kTileB + (j - 4) * 16 * kRowB),
-                                                 16, l.off_c, kb + (j - 4) * step, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            l.wgt, (__attribute__((address_space(3))) void *)(sb + kTileB + (l.wave * C::kChnRowsPerWave + (j - 4) * 16) * kRowB), 16,
+            l.off_c, kb + (j - 4) * step, 0, 0);
 }
+template <typename C>
 __device__ __forceinline__ void loader_end(Loader &l, Cursor &ld) {
     l.issued++;
     if (++ld.kt == l.nk) {
-        cursor_next_tile(ld);
-        if (ld.valid) loader_offsets(l, ld, fresh_lane_id()); else ld.kt = l.nk - 1;
+        cursor_next_tile<C>(ld);
+        if (ld.valid) loader_offsets<C>(l, ld, fresh_lane_id()); else ld.kt = l.nk - 1;
     }
 }
+template <typename C>
 __device__ __forceinline__ void loader_issue(Loader &l, Cursor &ld, uint8_t *lds) {
 #pragma unroll
-    for (int j = 0; j < kLoads; j++) loader_one(l, ld, lds, j);
-    loader_end(l, ld);
+    for (int j = 0; j < C::kLoads; j++) loader_one<C>(l, ld, lds, j);
+    loader_end<C>(l, ld);
 }
 
 template <int N>
@@ -603,8 +623,9 @@ __device__ __forceinline__ void wait_vmcnt_imm() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));   // vmcnt only
 }
 // at most kLoads * (kStages - 3) + extra younger memory operations may still be in flight
+template <typename C>
 __device__ __forceinline__ void wait_stage(int extra) {
-    constexpr int kBase = kLoads * (kStages - 3);
+    constexpr int kBase = C::kLoads * (C::kStages - 3);
     switch (extra) {
         case 36: wait_vmcnt_imm<kBase + 36>(); break;
         case 28: wait_vmcnt_imm<kBase + 28>(); break;
@@ -643,7 +664,7 @@ struct Frags {
 //   * `sync` runs after slot kSyncSlot (-1: none) and the stage's loads, dma(0..kLoads), follow one per few slots;
 //   * NEXT: the packed fragments of the next k-pair are read from LDS in the slots after that, up to 3/8 of the
 //     way, and split into `nxt` (3 VALU ops per dword) over the second half of the slots.
-template <int NA, bool NEXT, int kSyncSlot, typename Sync, typename Dma>
+template <typename C, int NA, bool NEXT, int kSyncSlot, typename Sync, typename Dma>
 __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Frags &cur, Frags &nxt, const uint8_t *rd_tok,
                                        const uint8_t *rd_chn, Sync &&sync, Dma &&dma) {
     constexpr int S = 8 * NA;                 // slots
@@ -663,7 +684,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
             // the stage's kLoads direct-to-LDS loads and the cursor step (item kLoads), spread over the remaining slots
             if (i > kSyncSlot) {
 #pragma unroll
-                for (int j = (i - R0) * (kLoads + 1) / (S - R0); j < (i - R0 + 1) * (kLoads + 1) / (S - R0); j++) dma(j);
+                for (int j = (i - R0) * (C::kLoads + 1) / (S - R0); j < (i - R0 + 1) * (C::kLoads + 1) / (S - R0); j++) dma(j);
             }
         }
         if constexpr (NEXT) {
@@ -686,7 +707,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
     }
 }
 
-template <int OUT, int NA>
+template <typename C, int OUT, int NA>
 __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, const int32_t *__restrict__ a_add,
                                          const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
                                          const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0,
@@ -720,7 +741,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
 
     // epilogue vectors of this tile -> LDS, also by direct loads: wave w brings 64 channels of b_add and b_mul
     // and 64 tokens of a_add and a_mul (four loads per wave, counted in pp.store_extra); read back after the K loop
-    uint8_t *vec = lds + kVecOff + pp.vec_par * kVecParB;
+    uint8_t *vec = lds + C::kVecOff + pp.vec_par * kVecParB;
     int32_t *v_add = reinterpret_cast<int32_t *>(vec);
     uint16_t *v_mul = reinterpret_cast<uint16_t *>(vec + kRows * 4);
     int32_t *w_add = reinterpret_cast<int32_t *>(vec + kRows * 6);
@@ -744,22 +765,22 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
 
     // ---- main loop: while one k-pair is multiplied the next is read from LDS and split ------------------------------
     // stage s = pp.it + kt; k-pair j of a stage is the 16-byte chunk 2 j + lg of each 64-byte stage row
-    auto tok_base = [&](int slot, int j) { return lds + slot * kStageB + rd_j[j] + rd_t; };
-    auto chn_base = [&](int slot, int j) { return lds + slot * kStageB + rd_j[j] + rd_c; };
+    auto tok_base = [&](int slot, int j) { return lds + slot * C::kStageB + rd_j[j] + rd_t; };
+    auto chn_base = [&](int slot, int j) { return lds + slot * C::kStageB + rd_j[j] + rd_c; };
     // stage s + 1 must have landed everywhere before its fragments are read; the slot of stage s - 1 is free for
     // the loads of stage s + kStages - 1 once everyone is past this barrier
     auto sync = [&]() {
-        if (pp.store_syncs > 0) { wait_stage(pp.store_extra); pp.store_syncs--; } else { wait_stage(0); }
+        if (pp.store_syncs > 0) { wait_stage<C>(pp.store_extra); pp.store_syncs--; } else { wait_stage<C>(0); }
         plain_barrier();
     };
-    auto dma = [&](int j) { if (j < kLoads) loader_one(ldr, ld, lds, j); else loader_end(ldr, ld); };
+    auto dma = [&](int j) { if (j < C::kLoads) loader_one<C>(ldr, ld, lds, j); else loader_end<C>(ldr, ld); };
     auto no_sync = []() {};
     if constexpr (NA == 0) {
-        for (int kt = 0; kt < nk; kt++) { sync(); loader_issue(ldr, ld, lds); pp.it++; }
+        for (int kt = 0; kt < nk; kt++) { sync(); loader_issue<C>(ldr, ld, lds); pp.it++; }
     } else {
         Frags u0, u1;
         {   // prologue: the first k-pair of the tile's first stage (landed: the previous synchronisation saw to it)
-            const int slot = pp.it % kStages;
+            const int slot = pp.it % C::kStages;
             const uint8_t *t0 = tok_base(slot, 0), *c0 = chn_base(slot, 0);
 #pragma unroll
             for (int f = 0; f < 4 + NA; f++) {
@@ -770,15 +791,15 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             }
         }
         for (int kt = 0; kt < nk - 1; kt++) {
-            const int slot = pp.it % kStages, next = (pp.it + 1) % kStages;
-            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
-            k_pair<NA, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync, dma);
+            const int slot = pp.it % C::kStages, next = (pp.it + 1) % C::kStages;
+            k_pair<C, NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
+            k_pair<C, NA, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync, dma);
             pp.it++;
         }
         {   // last stage of the tile: nothing of the next tile is read here (its channel rows sit elsewhere)
-            const int slot = pp.it % kStages;
-            k_pair<NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
-            k_pair<NA, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync, dma);
+            const int slot = pp.it % C::kStages;
+            k_pair<C, NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
+            k_pair<C, NA, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync, dma);
             pp.it++;
         }
     }
@@ -905,7 +926,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     // (the next tile's four vector loads, issued right after this point, are always exact)
     if constexpr (OUT != OUT_INT32) {
         pp.store_extra = (interior ? 8 * NA : 0) + 4;
-        pp.store_syncs = kStages - 2;
+        pp.store_syncs = C::kStages - 2;
     } else {
         pp.store_extra = 0;
         pp.store_syncs = 0;
@@ -913,13 +934,13 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     pp.vec_par ^= 1;
 }
 
-template <int OUT>
-__global__ void __launch_bounds__(256)
+template <typename C, int OUT>
+__global__ void __launch_bounds__(256, C::kWgPerCu)
 gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                      const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
                      const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
                      int M, int N, int K, stream::Schedule sch) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsB];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[C::kLdsB];
     // wave-uniform by construction; readfirstlane tells the compiler so, which keeps everything that is
     // updated under `switch (na)` below (cursors, slot numbers, LDS bases) in scalar registers; the empty
     // asm cuts the value loose from threadIdx, which would otherwise be kept (and spilled) to derive it again
@@ -947,9 +968,9 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     cc.valid = false;
     cc.tok0 = cc.ch0 = cc.width = cc.kt = 0;
     ld = cc;
-    cursor_next_tile(cc);
+    cursor_next_tile<C>(cc);
     if (!cc.valid) return;                       // uniform: the whole workgroup has nothing to do
-    cursor_next_tile(ld);
+    cursor_next_tile<C>(ld);
 
     Loader ldr;
     ldr.act = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, M * kbytes, 0x00020000);
@@ -962,33 +983,41 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     ldr.nk = K / 128;
     ldr.wave = wave;
     ldr.issued = 0;
-    loader_offsets(ldr, ld, fresh_lane_id());
+    loader_offsets<C>(ldr, ld, fresh_lane_id());
 
     // ---- pipeline prologue: stages 0 .. kStages - 2 in flight, stage 0 landed
 #pragma unroll
-    for (int s = 0; s < kStages - 1; s++) loader_issue(ldr, ld, lds);
-    wait_vmcnt_imm<kLoads * (kStages - 2)>();
+    for (int s = 0; s < C::kStages - 1; s++) loader_issue<C>(ldr, ld, lds);
+    wait_vmcnt_imm<C::kLoads * (C::kStages - 2)>();
     plain_barrier();
     Pipe pp;
     pp.it = 0;
     pp.store_extra = OUT != OUT_INT32 ? 4 : 0;   // the first tile's four vector loads
-    pp.store_syncs = OUT != OUT_INT32 ? kStages - 2 : 0;
+    pp.store_syncs = OUT != OUT_INT32 ? C::kStages - 2 : 0;
     pp.vec_par = 0;
     while (cc.valid) {
         const int h0 = (cc.width + 1) >> 1;
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
 #define QUEST_BIG_TILE(NA) \
-    big_tile<OUT, NA>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
-        switch (na) {
-            case 4: QUEST_BIG_TILE(4); break;
-            case 3: QUEST_BIG_TILE(3); break;
-            case 2: QUEST_BIG_TILE(2); break;
-            case 1: QUEST_BIG_TILE(1); break;
-            default: QUEST_BIG_TILE(0); break;
+    big_tile<C, OUT, NA>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
+        if constexpr (C::kMaxUnits > 4) {
+            switch (na) {
+                case 4: QUEST_BIG_TILE(4); break;
+                case 3: QUEST_BIG_TILE(3); break;
+                case 2: QUEST_BIG_TILE(2); break;
+                case 1: QUEST_BIG_TILE(1); break;
+                default: QUEST_BIG_TILE(0); break;
+            }
+        } else {
+            switch (na) {
+                case 2: QUEST_BIG_TILE(2); break;
+                case 1: QUEST_BIG_TILE(1); break;
+                default: QUEST_BIG_TILE(0); break;
+            }
         }
 #undef QUEST_BIG_TILE
-        cursor_next_tile(cc);
+        cursor_next_tile<C>(cc);
     }
     wait_vmcnt_imm<0>();                         // no direct-to-LDS load may outlive the workgroup's LDS allocation
 }
@@ -1022,17 +1051,17 @@ static int gemm_launch_stream(void *out, const uint8_t *a, const uint8_t *b, con
     return launch_status();
 }
 
-template <int OUT>
+template <typename C, int OUT>
 static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                            const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
     stream::Schedule sch;
     sch.tiles_t = (M + big::kRows - 1) / big::kRows;
     sch.units = (N + 31) / 32;
     const long cells = (long)sch.tiles_t * sch.units;
-    long grid = device_cu_count();                          // one workgroup per CU
+    long grid = (long)C::kWgPerCu * device_cu_count();      // persistent: one or two workgroups per CU
     if (grid > cells) grid = cells;
     sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
-    big::gemm_w4a4_big_kernel<OUT><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+    big::gemm_w4a4_big_kernel<C, OUT><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
         out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
     return launch_status();
 }
@@ -1047,7 +1076,11 @@ static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int3
     }
     // the large-tile kernel fetches the 16-bit scale vectors two per dword: even M, N and 4-byte aligned vectors
     if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && (M & 1) == 0 && aligned(b_mul, 4) && aligned(a_mul, 4))
-        return gemm_launch_big<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    {
+        // the wide shape pays off when most of its tiles are full width: 16 or more channel units per XCD group
+        if (N >= 4096) return gemm_launch_big<big::Wide, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        return gemm_launch_big<big::Duo, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    }
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
