@@ -641,6 +641,8 @@ struct Pipe {            // state that lives across tiles
     int store_extra;     // epilogue stores that may still be in flight ...
     int store_syncs;     // ... for this many more stage synchronisations
     int vec_par;
+    unsigned clock;      // two workgroups per CU: the cycle counter sampled at the previous stage synchronisation ...
+    int half;            // ... and which half of the grid this workgroup is in (see `sync` in big_tile)
 };
 
 __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
@@ -772,6 +774,14 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     auto sync = [&]() {
         if (pp.store_syncs > 0) { wait_stage<C>(pp.store_extra); pp.store_syncs--; } else { wait_stage<C>(0); }
         plain_barrier();
+        if constexpr (C::kWgPerCu > 1) {
+            // Two persistent workgroups share each SIMD and the issue arbiter prefers the older wave: left alone, the
+            // workgroup launched first runs at nearly full speed, finishes a third early and leaves the other to run
+            // the rest by itself, without anything to overlap its waits.  Alternating the wave priority between the
+            // two halves of the grid in windows of 2^14 cycles (a few stages) keeps them level.
+            if ((((pp.clock >> 14) ^ pp.half) & 1) != 0) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
+            pp.clock = (unsigned)__builtin_amdgcn_s_memtime();       // read one stage later: never waited for
+        }
     };
     auto dma = [&](int j) { if (j < C::kLoads) loader_one<C>(ldr, ld, lds, j); else loader_end<C>(ldr, ld); };
     auto no_sync = []() {};
@@ -995,6 +1005,8 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     pp.store_extra = OUT != OUT_INT32 ? 4 : 0;   // the first tile's four vector loads
     pp.store_syncs = OUT != OUT_INT32 ? C::kStages - 2 : 0;
     pp.vec_par = 0;
+    pp.clock = 0;
+    pp.half = blockIdx.x >= gridDim.x / 2 ? 1 : 0;
     while (cc.valid) {
         const int h0 = (cc.width + 1) >> 1;
         const int na = wc == 0 ? h0 : cc.width - h0;
