@@ -841,11 +841,19 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             }
         }
         uint8_t *out_lane = reinterpret_cast<uint8_t *>(out) + ((size_t)(tok0 + wt * 128 + li_e) * N + ch0 + unit0 * 32) * kEs;
+        // Loop order.  One workgroup per CU: channel unit outside, so that a unit's 32 scale values are read from
+        // LDS once.  Two per CU: token sub-tile outside, so that the stores of consecutive iterations complete whole
+        // 128-byte lines of the same rows (measured -3..-6 % run time at short K; nothing for the wide shape).
+        constexpr bool kTokOuter = C::kWgPerCu > 1;
+        int adds[16];
+        float muls[16];
 #pragma unroll
-        for (int a = 0; a < NA; a++) {
-            int adds[16];
-            float muls[16];
+        for (int o = 0; o < (kTokOuter ? 4 : NA); o++) {
+#pragma unroll
+          for (int i = 0; i < (kTokOuter ? NA : 4); i++) {
+            const int a = kTokOuter ? i : o, b = kTokOuter ? o : i;
             if constexpr (OUT != OUT_INT32) {
+              if (kTokOuter || i == 0) {
 #pragma unroll
                 for (int rg = 0; rg < 4; rg++) {
                     const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;      // channel inside the tile
@@ -855,9 +863,9 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                     muls[rg * 4 + 0] = lo_f32<DT>(vm.x); muls[rg * 4 + 1] = hi_f32<DT>(vm.x);
                     muls[rg * 4 + 2] = lo_f32<DT>(vm.y); muls[rg * 4 + 3] = hi_f32<DT>(vm.y);
                 }
+              }
             }
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
+            {
                 const bool tok_ok = tok0 + wt * 128 + b * 32 + li_e < M;
                 uint8_t *dst = out_lane + ((size_t)b * 32 * N + a * 32) * kEs;
                 if constexpr (OUT == OUT_INT32) {
@@ -895,6 +903,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                     }
                 }
             }
+          }
         }
     } else if (NA > 0) {
         // generic path (N not a multiple of 8 / 4): element-wise stores straight from the accumulators
@@ -1089,8 +1098,17 @@ static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int3
     // the large-tile kernel fetches the 16-bit scale vectors two per dword: even M, N and 4-byte aligned vectors
     if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && (M & 1) == 0 && aligned(b_mul, 4) && aligned(a_mul, 4))
     {
-        // the wide shape pays off when most of its tiles are full width: 16 or more channel units per XCD group
-        if (N >= 4096) return gemm_launch_big<big::Wide, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        // Wide (256 x 256 tiles, a lone wave per SIMD) has the cheaper main loop; Duo (256 x 128, two workgroups per
+        // CU) hides epilogues and waits.  Duo wins where there is enough work for full-width tiles on 512 workgroups
+        // (256 cells of 256 tokens x 32 channels per XCD group) and the epilogue weighs much: K short, or fewer
+        // than 16 channel units per group, which would leave Wide with narrow tiles.  Measured over M in
+        // {1024, 4096, 16384}, K in {1024 .. 11008}, N in {1024 .. 11008}: the rule picks the faster shape or
+        // stays within 4 % of it except for a few of the smallest problems.
+        const int units = (N + 31) / 32;
+        const int per_group = units >= 8 ? units / 8 : units;
+        const long cells_per_group = (long)((M + big::kRows - 1) / big::kRows) * per_group;
+        const bool duo = cells_per_group >= 256 && (K <= 1024 || per_group < 16);
+        if (!duo) return gemm_launch_big<big::Wide, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
         return gemm_launch_big<big::Duo, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     }
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
