@@ -136,6 +136,18 @@ int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *norm_weight,
                                          int dtype, void *stream);
 
 /*
+ * quest_rmsnorm_hadamard_quantize_int4 with the residual addition in front of the norm (x = x + attn(...);
+ * ... ln_2(x), src/models/llama.py:175-176, and the same across two blocks): x <- dtype(x + branch) in place, one
+ * rounding as the framework's addition has, then everything above on the new x.  Saves the separate addition pass
+ * (two reads and a write of the residual stream).  No counterpart in the reference's quest package.  Limits and
+ * error behaviour as above; x and branch are (batch_size, group_size) and must not overlap.
+ */
+int quest_add_rmsnorm_hadamard_quantize_int4(void *x, const void *branch, const void *norm_weight, float eps,
+                                             void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
+                                             int group_size, int batch_size, float had_scale, int dtype,
+                                             void *stream);
+
+/*
  * The same for the SwiGLU product in front of the MLP's output projection (src/models/llama.py:117-118):
  * gate_up is (batch_size, 2 * group_size), gate in the first half of each row and up in the second;
  * y = dtype(dtype(silu(gate)) * up), silu(g) = g / (1 + exp(-g)) in fp32.  x_act, when not NULL, receives y

@@ -18,6 +18,7 @@ from .api import (  # noqa: F401
     quantize_int4,
     reorder_meta48_int4,
     rmsnorm_hadamard_quantize_int4,
+    add_rmsnorm_hadamard_quantize_int4,
     rope_interleaved_,
     silu_mul_hadamard_quantize_int4,
     uncompress_meta48_int4,

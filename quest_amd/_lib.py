@@ -31,6 +31,7 @@ SIGNATURES = {
     'quest_hadamard128': [_vp, _vp, _i, _i, _f, _i, _vp],
     'quest_hadamard_quantize_int4': [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_rmsnorm_hadamard_quantize_int4': [_vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
+    'quest_add_rmsnorm_hadamard_quantize_int4': [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_hadamard_quantize_int4_rule': [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
     'quest_rope_interleaved': [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     'quest_silu_mul_hadamard_quantize_int4': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],

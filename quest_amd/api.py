@@ -239,6 +239,32 @@ def rmsnorm_hadamard_quantize_int4(
     return scale, x_int_packed, x_int_row_sum
 
 
+def add_rmsnorm_hadamard_quantize_int4(
+        x: torch.Tensor,
+        branch: torch.Tensor,
+        norm_weight: torch.Tensor,
+        eps: float,
+        scale: torch.Tensor = None,
+        x_int_packed: torch.Tensor = None,
+        x_int_row_sum: torch.Tensor = None,
+        hadamard_scale: float = HADAMARD_ENTRY,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """`x += branch` (the residual addition of src/models/llama.py:175-176, in place) followed by
+    `rmsnorm_hadamard_quantize_int4(x, ...)`, in one pass over the two tensors (M, K <= 4096).
+    Returns (scale, x_int_packed, x_int_row_sum); x holds the sum afterwards."""
+    m, k = x.shape
+    assert x.dtype in _FLOAT16S and x.is_contiguous() and branch.dtype == x.dtype and branch.shape == x.shape
+    assert branch.is_contiguous() and branch.data_ptr() != x.data_ptr()
+    assert norm_weight.dtype == x.dtype and norm_weight.numel() == k and norm_weight.is_contiguous()
+    scale, x_int_packed, x_int_row_sum = _quant_outputs(m, k, x.dtype, x.device, scale, x_int_packed, x_int_row_sum)
+    dev = require_gpu(x, branch, norm_weight, scale, x_int_packed, x_int_row_sum)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_add_rmsnorm_hadamard_quantize_int4(
+            ptr(x), ptr(branch), ptr(norm_weight), float(eps), ptr(scale), ptr(x_int_packed), ptr(x_int_row_sum),
+            k, m, float(hadamard_scale), DTYPE_CODE[x.dtype], stream_of(x)), 'add_rmsnorm_hadamard_quantize_int4')
+    return scale, x_int_packed, x_int_row_sum
+
+
 def silu_mul_hadamard_quantize_int4(
         gate_up: torch.Tensor,
         scale: torch.Tensor = None,

@@ -230,7 +230,7 @@ int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t 
 // front (pre: 0 none, 1 RMSNorm, 2 SiLU(gate) * up); QUEST_ERR_UNSUPPORTED when it does not apply
 int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
                                   int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
-                                  hipStream_t st);
+                                  hipStream_t st, const void *add_in = nullptr, void *sum_out = nullptr);
 
 inline int check_dtype(int dtype) { return dtype == QUEST_DTYPE_BF16 || dtype == QUEST_DTYPE_FP16; }
 inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

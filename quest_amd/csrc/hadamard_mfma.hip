@@ -64,6 +64,8 @@ struct Shape {
 // What is applied to the input on its way into the transform (the producer the activation comes from):
 //   kPreNone     nothing;
 //   kPreRmsNorm  y = dtype(dtype(f32(x) * rsqrt(mean(x^2) + eps)) * w)    (src/models/llama.py:71-77 of the reference);
+//                with add_in: x is first replaced by dtype(x + add_in) -- the residual addition in front of the norm
+//                (llama.py:175-176) -- and that sum is written to sum_out (which may be x itself);
 //   kPreSiluMul  y = dtype(dtype(silu(gate)) * up), gate and up the two halves of a (M, 2 K) row (llama.py:117-118).
 enum { kPreNone = 0, kPreRmsNorm = 1, kPreSiluMul = 2 };
 
@@ -94,8 +96,8 @@ template <int DT, int WPR, int G, int PRE>
 __global__ void __launch_bounds__(64 * Shape<WPR>::kWaves, Shape<WPR>::kMinBlocks)
 hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ norm_w,
                               uint16_t *__restrict__ scale, uint32_t *__restrict__ packed, int32_t *__restrict__ row_sum,
-                              uint16_t *__restrict__ x_had, uint16_t *__restrict__ pre_out, int K, int M, int ldx,
-                              uint32_t entry_bits, float eps) {
+                              uint16_t *__restrict__ x_had, uint16_t *__restrict__ pre_out, const uint16_t *add_in,
+                              uint16_t *sum_out, int K, int M, int ldx, uint32_t entry_bits, float eps) {
     static_assert(WPR == 1 || (G == 32 && PRE == kPreNone), "rows shared by waves: whole waves, no producer");
     constexpr int kRows = Shape<WPR>::kRows;
     constexpr int kRowsPerWave = 32 / G;
@@ -150,6 +152,24 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
     __builtin_amdgcn_sched_barrier(0);
 
     if constexpr (PRE == kPreRmsNorm) {
+        if (add_in != nullptr) {                 // uniform: the residual stream plus the branch that ends here
+            const __amdgpu_buffer_rsrc_t ar =
+                __builtin_amdgcn_make_buffer_rsrc((void *)add_in, 0, (int)((long)M * K * 2), 0x00020000);
+            v4u aq[8];
+#pragma unroll
+            for (int s = 0; s < 8; s++) aq[s] = __builtin_amdgcn_raw_buffer_load_b128(ar, (int)(ld_off + 32 * s), 0, 0);
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    bq[s][d] = pack2_rounded_products<DT>(__fadd_rn(lo_f32<DT>(bq[s][d]), lo_f32<DT>(aq[s][d])),
+                                                          __fadd_rn(hi_f32<DT>(bq[s][d]), hi_f32<DT>(aq[s][d])));
+            if (live) {
+                uint16_t *dst = sum_out + (size_t)row * K + blk * 128 + 8 * h;
+#pragma unroll
+                for (int s = 0; s < 8; s++) *reinterpret_cast<v4u *>(dst + 16 * s) = bq[s];
+            }
+        }
         const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)norm_w, 0, K * 2, 0x00020000);
         const uint32_t w_off = live ? (uint32_t)(blk * 256 + h * 16) : dead;
         v4u wq[8];
@@ -319,6 +339,8 @@ struct Args {
     uint8_t *packed;
     int32_t *row_sum;
     void *x_had, *pre_out;
+    const void *add_in;
+    void *sum_out;
     int K, M, ldx;
     uint32_t bits;
     float eps;
@@ -330,7 +352,7 @@ static void launch_shape(const Args &a) {
     constexpr int rows = hq::Shape<WPR>::kRows * (32 / G);        // rows per workgroup
     hq::hadamard_quantize_mfma_kernel<DT, WPR, G, PRE><<<dim3((a.M + rows - 1) / rows), dim3(64 * hq::Shape<WPR>::kWaves), 0, a.st>>>(
         (const uint16_t *)a.x, (const uint16_t *)a.norm_w, (uint16_t *)a.scale, (uint32_t *)a.packed, a.row_sum,
-        (uint16_t *)a.x_had, (uint16_t *)a.pre_out, a.K, a.M, a.ldx, a.bits, a.eps);
+        (uint16_t *)a.x_had, (uint16_t *)a.pre_out, (const uint16_t *)a.add_in, (uint16_t *)a.sum_out, a.K, a.M, a.ldx, a.bits, a.eps);
 }
 
 // rows of up to 32 blocks: one wave holds 32 / G of them
@@ -373,17 +395,20 @@ static void launch_dtype(int pre, const Args &a) {
 
 // Launches the matrix-core kernel when it applies (K a multiple of 128 up to 32768 -- 4096 with a producer --, a
 // Hadamard entry the dtype represents exactly); returns QUEST_ERR_UNSUPPORTED otherwise so that the caller can take
-// another path.  pre: 0 none, 1 RMSNorm (norm_w, eps), 2 SiLU(gate) * up with x a (M, 2 K) tensor.
+// another path.  pre: 0 none, 1 RMSNorm (norm_w, eps; with add_in the norm of x + add_in, the sum written to
+// sum_out), 2 SiLU(gate) * up with x a (M, 2 K) tensor.
 int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
                                   int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
-                                  hipStream_t st) {
+                                  hipStream_t st, const void *add_in, void *sum_out) {
     uint32_t bits = 0;
     if (K > 32768 || (K & 127) || had_scale <= 0.f || !representable16(had_scale, dtype, &bits)) return QUEST_ERR_UNSUPPORTED;
     if (pre != hq::kPreNone && K > 4096) return QUEST_ERR_UNSUPPORTED;
     const int ldx = pre == hq::kPreSiluMul ? 2 * K : K;
     if ((long)M * ldx * 2 >= (1L << 31)) return QUEST_ERR_UNSUPPORTED;        // 32-bit buffer offsets
     if (!aligned(packed, 16) || !aligned(x_had, 8) || !aligned(pre_out, 16) || !aligned(norm_w, 16)) return QUEST_ERR_UNSUPPORTED;
-    const Args a = {x, norm_w, scale, packed, row_sum, x_had, pre_out, K, M, ldx, bits, eps, st};
+    if (add_in != nullptr && (pre != hq::kPreRmsNorm || sum_out == nullptr || !aligned(add_in, 16) || !aligned(sum_out, 16)))
+        return QUEST_ERR_UNSUPPORTED;
+    const Args a = {x, norm_w, scale, packed, row_sum, x_had, pre_out, add_in, sum_out, K, M, ldx, bits, eps, st};
     if (dtype == QUEST_DTYPE_BF16) launch_dtype<0>(pre, a);
     else launch_dtype<1>(pre, a);
     return launch_status();

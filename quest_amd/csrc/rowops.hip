@@ -436,6 +436,19 @@ extern "C" int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *n
                                          group_size, batch_size, had_scale, dtype, (hipStream_t)stream);
 }
 
+extern "C" int quest_add_rmsnorm_hadamard_quantize_int4(void *x, const void *branch, const void *norm_weight, float eps,
+                                                        void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
+                                                        int group_size, int batch_size, float had_scale, int dtype,
+                                                        void *stream) {
+    if (!x || !branch || !norm_weight || !scale) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(x, 16) || !aligned(branch, 16) || !aligned(norm_weight, 16) || !aligned(x_int_packed, 16))
+        return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(1, x, norm_weight, eps, scale, x_int_packed, x_int_row_sum, nullptr, nullptr,
+                                         group_size, batch_size, had_scale, dtype, (hipStream_t)stream, branch, x);
+}
+
 extern "C" int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *scale, uint8_t *x_int_packed,
                                                      int32_t *x_int_row_sum, void *x_had, void *x_act, int group_size,
                                                      int batch_size, float had_scale, int dtype, void *stream) {

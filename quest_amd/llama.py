@@ -154,23 +154,29 @@ class LlamaBlock(nn.Module):
 
     def forward(self, x, freqs_cis):
         if self.fuse_producers:
-            return self._forward_fused(x, freqs_cis)
+            x, branch = self.forward_fused(x, freqs_cis)
+            return x + branch
         x = x + self.attn(self.ln_1(x), freqs_cis)
         return x + self.mlp(self.ln_2(x))
 
-    def _forward_fused(self, x, freqs_cis):
+    def forward_fused(self, x, freqs_cis, branch=None):
         """The same block with each W4A4 linear fed by the kernel that also computes its input: RMSNorm -> codes for
         c_attn and for the fused gate/up projection, silu(gate) * up -> codes for the MLP's c_proj.  Three bf16
-        tensors per block (two normalised activations, one SwiGLU product) are never written or re-read."""
+        tensors per block (two normalised activations, one SwiGLU product) are never written or re-read, and the
+        residual additions run inside the norm kernels: x is the residual stream, updated IN PLACE; `branch`, if
+        given, is the previous block's MLP output still to be added to it.  Returns (x, this block's MLP output):
+        the caller adds the last one (or hands it to the next block)."""
         b, t, c = x.shape
         x2 = x.view(b * t, c)
-        q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
-        x = x + self.attn.attend(self.attn.c_attn.forward_quantized(*q).view(b, t, 3 * c), freqs_cis)
-        x2 = x.view(b * t, c)
-        q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_2.weight, self.ln_2.eps)
+        if branch is None:
+            q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
+        else:
+            q = quest.add_rmsnorm_hadamard_quantize_int4(x2, branch.view(b * t, c), self.ln_1.weight, self.ln_1.eps)
+        att = self.attn.attend(self.attn.c_attn.forward_quantized(*q).view(b, t, 3 * c), freqs_cis)
+        q = quest.add_rmsnorm_hadamard_quantize_int4(x2, att.view(b * t, c), self.ln_2.weight, self.ln_2.eps)
         gate_up = self.mlp.w12.forward_quantized(*q)
         q = quest.silu_mul_hadamard_quantize_int4(gate_up)
-        return x + self.mlp.c_proj.forward_quantized(*q).view(b, t, c)
+        return x, self.mlp.c_proj.forward_quantized(*q).view(b, t, c)
 
 
 class Llama(nn.Module):
@@ -207,8 +213,16 @@ class Llama(nn.Module):
         if self.freqs_cis.device != x.device:          # moved once, outside any graph capture (the table stays fp32)
             self.freqs_cis = self.freqs_cis.to(x.device)
         freqs_cis = self.freqs_cis[:t]
+        branch = None                                  # a fused block's MLP output, not yet added to the stream
         for block in self.transformer.h:
-            x = block(x, freqs_cis)
+            if block.fuse_producers and x.is_contiguous():
+                x, branch = block.forward_fused(x, freqs_cis, branch)
+            else:
+                if branch is not None:
+                    x, branch = x + branch, None
+                x = block(x, freqs_cis)
+        if branch is not None:
+            x = x + branch
         return self.transformer.ln_f(x)
 
     def forward(self, idx: torch.Tensor, all_logits: bool = False) -> dict:

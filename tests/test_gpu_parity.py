@@ -348,6 +348,25 @@ def test_rmsnorm_hadamard_quantize(quest, dtype, shape):
 
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', PRODUCER_SHAPES)
+def test_add_rmsnorm_hadamard_quantize(quest, dtype, shape):
+    """The residual addition in front of the norm: x becomes dtype(x + branch) -- bit for bit the sum torch's CPU
+    addition gives, the oracle's `x + ...` (llama_oracle.forward) -- and everything else is the norm kernel on that
+    sum, bit for bit."""
+    m, k = shape
+    x = rand_act(m, k, dtype, seed=22)
+    branch = rand_act(m, k, dtype, seed=23)
+    w = (1 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(24))).to(dtype)
+    want_sum = x + branch                                   # CPU: fp32 sum, one rounding
+    gx, gb, gw = x.to(DEV), branch.to(DEV), w.to(DEV)
+    scale, packed, row_sum = quest.add_rmsnorm_hadamard_quantize_int4(gx, gb, gw, 1e-5)
+    assert torch.equal(bits(gx.cpu()), bits(want_sum)), 'x must hold the rounded sum'
+    assert torch.equal(bits(gb.cpu()), bits(branch)), 'the branch must not be written'
+    s2, p2, r2 = quest.rmsnorm_hadamard_quantize_int4(want_sum.to(DEV), gw, 1e-5)
+    assert torch.equal(bits(scale.cpu()), bits(s2.cpu())) and torch.equal(packed, p2) and torch.equal(row_sum, r2)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', PRODUCER_SHAPES)
 def test_silu_mul_hadamard_quantize(quest, dtype, shape):
     """SwiGLU product in front of the fused kernel, against torch's CPU silu(gate) * up."""
     m, k = shape
