@@ -122,6 +122,21 @@ int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uint8_t *x_int
                                       int scale_rule, int dtype, void *stream);
 
 /*
+ * quest_fused_matmul_dequantize_int4_int4t for the gate and up projections of a SwiGLU MLP in one GEMM, with the
+ * gated unit applied in the epilogue: mat_b holds the 2 H weight rows interleaved in eights -- rows 8 g .. 8 g + 3
+ * the gate rows of outputs 4 g .. 4 g + 3, rows 8 g + 4 .. 8 g + 7 their up rows -- with vec_b_add / vec_b_mul in the
+ * same order, and mat_d (size_m, size_n / 2) = dtype(dtype(silu(gate)) * up), gate and up being the two
+ * dtype-rounded outputs the plain entry point would have written (silu(g) = g / (1 + exp(-g)) in fp32;
+ * src/models/llama.py:117-118).  The (size_m, 2 H) tensor is never written.  No counterpart in the reference, which
+ * runs two GEMMs and the torch expression.  size_n % 8 == 0; QUEST_ERR_UNSUPPORTED unless size_k % 128 == 0,
+ * size_m > 64 and even (the caller then uses the plain entry point and applies the unit itself).
+ */
+int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                    const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                    const void *vec_a_mul, const void *vec_b_mul, int size_m,
+                                                    int size_k, int size_n, int dtype, void *stream);
+
+/*
  * quest_hadamard_quantize_int4 with the producer of the activation in front, so that the normalised tensor is
  * never written: y = dtype(dtype(f32(x) * rsqrt(mean(x^2) + eps)) * norm_weight) -- the RMSNorm in front of every
  * attention and MLP block of the reference's model (src/models/llama.py:71-77, applied at llama.py:174-175) --

@@ -10,6 +10,8 @@ from .api import (  # noqa: F401
     find_scale_int4,
     fused_matmul_dequantize_int4_int4t,
     fused_matmul_dequantize_int4_int4t_bf16,
+    fused_matmul_dequantize_swiglu_int4_int4t,
+    swiglu_interleave_rows,
     generate_random_meta48_int4,
     hadamard128,
     hadamard_quantize_int4,

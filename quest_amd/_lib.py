@@ -28,6 +28,7 @@ SIGNATURES = {
     'quest_add_mul_vv': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     'quest_matmul_int4_int4t_int32': [_vp, _vp, _vp, _i, _i, _i, _vp],
     'quest_fused_matmul_dequantize_int4_int4t': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    'quest_fused_matmul_dequantize_swiglu_int4_int4t': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     'quest_hadamard128': [_vp, _vp, _i, _i, _f, _i, _vp],
     'quest_hadamard_quantize_int4': [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_rmsnorm_hadamard_quantize_int4': [_vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],

@@ -48,6 +48,44 @@ def fused_matmul_dequantize_int4_int4t_bf16(
 fused_matmul_dequantize_int4_int4t = fused_matmul_dequantize_int4_int4t_bf16
 
 
+def swiglu_interleave_rows(n_out: int, device=None) -> torch.Tensor:
+    """Row order `fused_matmul_dequantize_swiglu_int4_int4t` expects of a (2 H, ...) gate-over-up weight stack: the
+    index tensor p with stacked[p] = rows in eights, four gate rows followed by the four up rows of the same outputs."""
+    assert n_out % 4 == 0
+    g = torch.arange(n_out, device=device).view(-1, 1, 4)
+    return torch.cat((g, g + n_out), dim=1).reshape(-1)
+
+
+def fused_matmul_dequantize_swiglu_int4_int4t(
+        mat_a: torch.Tensor,
+        mat_b: torch.Tensor,
+        vec_a_add: torch.Tensor,
+        vec_b_add: torch.Tensor,
+        vec_a_mul: torch.Tensor,
+        vec_b_mul: torch.Tensor,
+        out: torch.Tensor = None,
+) -> torch.Tensor:
+    """The gate/up GEMM of a SwiGLU MLP with `silu(gate) * up` (src/models/llama.py:117-118 of the reference) applied
+    in its epilogue: mat_b (2 H, K/2) and the vec_b_* hold the rows in `swiglu_interleave_rows` order; returns (M, H).
+    Raises RuntimeError (QUEST_ERR_UNSUPPORTED) for M <= 64, odd M or K % 128 != 0."""
+    m, n = mat_a.size(0), mat_b.size(0)
+    if out is None:
+        out = torch.empty(m, n // 2, dtype=vec_a_mul.dtype, device=mat_a.device)
+    assert mat_a.dtype == torch.uint8 and mat_b.dtype == torch.uint8 and vec_a_add.dtype == torch.int32 and vec_b_add.dtype == torch.int32
+    assert vec_a_mul.dtype in _FLOAT16S and vec_b_mul.dtype == vec_a_mul.dtype and out.dtype == vec_a_mul.dtype
+    for t in (mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, out):
+        assert t.is_contiguous()
+    assert mat_a.size(1) == mat_b.size(1) and vec_a_add.numel() == m and vec_a_mul.numel() == m
+    assert vec_b_add.numel() == n and vec_b_mul.numel() == n and n % 8 == 0 and out.shape == (m, n // 2)
+    dev = require_gpu(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, out)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_fused_matmul_dequantize_swiglu_int4_int4t(
+            ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
+            m, mat_b.size(1) * 2, n, DTYPE_CODE[out.dtype], stream_of(out)),
+            'fused_matmul_dequantize_swiglu_int4_int4t')
+    return out
+
+
 def matmul_int4_int4t_int32(
         mat_a: torch.Tensor,
         mat_b: torch.Tensor,

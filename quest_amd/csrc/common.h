@@ -70,6 +70,16 @@ __device__ __forceinline__ uint32_t pack2_rounded_products(float lo, float hi) {
     return pack2_rne<DT>(lo, hi);
 }
 
+// SwiGLU on two packed 16-bit pairs: dtype(dtype(silu(gate)) * up), silu(g) = g / (1 + exp(-g)) in fp32 (fast
+// exponential and reciprocal), as src/models/llama.py:117-118 of the reference rounds it.  One definition for the
+// activation kernel and the GEMM epilogue, so that the two agree bit for bit.
+template <int DT>
+__device__ __forceinline__ uint32_t silu_mul_pair(uint32_t gate2, uint32_t up2) {
+    auto silu = [](float g) { return __fdividef(g, 1.0f + __expf(-g)); };
+    const uint32_t a = pack2_rounded_products<DT>(silu(lo_f32<DT>(gate2)), silu(hi_f32<DT>(gate2)));
+    return pack2_rounded_products<DT>(__fmul_rn(lo_f32<DT>(a), lo_f32<DT>(up2)), __fmul_rn(hi_f32<DT>(a), hi_f32<DT>(up2)));
+}
+
 // ---- cross-lane moves -----------------------------------------------------------------------
 // value of lane (lane ^ M); M = 1, 2, 8 are single DPP moves, 4 and 16 LDS-crossbar swizzles.
 template <int M>

@@ -709,7 +709,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
     }
 }
 
-template <typename C, int OUT, int NA>
+template <typename C, int OUT, bool GLU, int NA>
 __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, const int32_t *__restrict__ a_add,
                                          const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
                                          const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0,
@@ -840,7 +840,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                 t_half_mul[b] = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
             }
         }
-        uint8_t *out_lane = reinterpret_cast<uint8_t *>(out) + ((size_t)(tok0 + wt * 128 + li_e) * N + ch0 + unit0 * 32) * kEs;
+        // GLU: the output has N / 2 columns, 16 per channel unit (see the store below)
+        constexpr int kOutPerUnit = GLU ? 16 : 32;
+        const int n_out = GLU ? N >> 1 : N;
+        uint8_t *out_lane = reinterpret_cast<uint8_t *>(out) +
+                            ((size_t)(tok0 + wt * 128 + li_e) * n_out + (size_t)((ch0 >> 5) + unit0) * kOutPerUnit) * kEs;
         // Loop order.  One workgroup per CU: channel unit outside, so that a unit's 32 scale values are read from
         // LDS once.  Two per CU: token sub-tile outside, so that the stores of consecutive iterations complete whole
         // 128-byte lines of the same rows (measured -3..-6 % run time at short K; nothing for the wide shape).
@@ -867,7 +871,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             }
             {
                 const bool tok_ok = tok0 + wt * 128 + b * 32 + li_e < M;
-                uint8_t *dst = out_lane + ((size_t)b * 32 * N + a * 32) * kEs;
+                uint8_t *dst = out_lane + ((size_t)b * 32 * n_out + a * kOutPerUnit) * kEs;
                 if constexpr (OUT == OUT_INT32) {
 #pragma unroll
                     for (int rg = 0; rg < 4; rg++) {
@@ -898,14 +902,22 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                         const auto s0 = __builtin_amdgcn_permlane32_swap(x[2 * pr][0], x[2 * pr + 1][0], false, false);
                         const auto s1 = __builtin_amdgcn_permlane32_swap(x[2 * pr][1], x[2 * pr + 1][1], false, false);
                         const int cl = (unit0 + a) * 32 + (2 * pr + lg_e) * 8;
-                        if (tok_ok && ch0 + cl < N)
+                        if constexpr (GLU) {
+                            // The weight rows come interleaved in eights, four gate rows then the four up rows of the same
+                            // outputs: after the swap a lane holds exactly such an eight, gates in (s0[0], s1[0]), ups in
+                            // (s0[1], s1[1]), and stores dtype(dtype(silu(gate)) * up) for its four outputs.
+                            if (tok_ok && ch0 + cl < N)
+                                *reinterpret_cast<uint2 *>(dst + (2 * pr + lg_e) * 8) =
+                                    make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
+                        } else if (tok_ok && ch0 + cl < N) {
                             *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                        }
                     }
                 }
             }
           }
         }
-    } else if (NA > 0) {
+    } else if (NA > 0 && !GLU) {
         // generic path (N not a multiple of 8 / 4): element-wise stores straight from the accumulators
 #pragma unroll
         for (int b = 0; b < 4; b++) {
@@ -953,7 +965,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     pp.vec_par ^= 1;
 }
 
-template <typename C, int OUT>
+template <typename C, int OUT, bool GLU>
 __global__ void __launch_bounds__(256, C::kWgPerCu)
 gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                      const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
@@ -1021,7 +1033,7 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
 #define QUEST_BIG_TILE(NA) \
-    big_tile<C, OUT, NA>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
+    big_tile<C, OUT, GLU, NA>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
         if constexpr (C::kMaxUnits > 4) {
             switch (na) {
                 case 4: QUEST_BIG_TILE(4); break;
@@ -1072,7 +1084,7 @@ static int gemm_launch_stream(void *out, const uint8_t *a, const uint8_t *b, con
     return launch_status();
 }
 
-template <typename C, int OUT>
+template <typename C, int OUT, bool GLU = false>
 static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                            const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
     stream::Schedule sch;
@@ -1082,9 +1094,26 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
     long grid = (long)C::kWgPerCu * device_cu_count();      // persistent: one or two workgroups per CU
     if (grid > cells) grid = cells;
     sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
-    big::gemm_w4a4_big_kernel<C, OUT><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+    big::gemm_w4a4_big_kernel<C, OUT, GLU><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
         out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
     return launch_status();
+}
+
+// Wide (256 x 256 tiles, a lone wave per SIMD) has the cheaper main loop; Duo (256 x 128, two workgroups per CU)
+// hides epilogues and waits.  Duo wins where there is enough work for full-width tiles on 512 workgroups (256 cells
+// of 256 tokens x 32 channels per XCD group) and the epilogue weighs much: K short, or fewer than 16 channel units
+// per group, which would leave Wide with narrow tiles.  Measured over M in {1024, 4096, 16384}, K in {1024 .. 11008},
+// N in {1024 .. 11008}: the rule picks the faster shape or stays within 4 % of it except for a few of the smallest
+// problems.
+template <int OUT, bool GLU>
+static int gemm_launch_large(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
+                             const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    const int units = (N + 31) / 32;
+    const int per_group = units >= 8 ? units / 8 : units;
+    const long cells_per_group = (long)((M + big::kRows - 1) / big::kRows) * per_group;
+    const bool duo = cells_per_group >= 256 && (K <= 1024 || per_group < 16);
+    if (!duo) return gemm_launch_big<big::Wide, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    return gemm_launch_big<big::Duo, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
 
 template <int OUT>
@@ -1097,20 +1126,7 @@ static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int3
     }
     // the large-tile kernel fetches the 16-bit scale vectors two per dword: even M, N and 4-byte aligned vectors
     if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && (M & 1) == 0 && aligned(b_mul, 4) && aligned(a_mul, 4))
-    {
-        // Wide (256 x 256 tiles, a lone wave per SIMD) has the cheaper main loop; Duo (256 x 128, two workgroups per
-        // CU) hides epilogues and waits.  Duo wins where there is enough work for full-width tiles on 512 workgroups
-        // (256 cells of 256 tokens x 32 channels per XCD group) and the epilogue weighs much: K short, or fewer
-        // than 16 channel units per group, which would leave Wide with narrow tiles.  Measured over M in
-        // {1024, 4096, 16384}, K in {1024 .. 11008}, N in {1024 .. 11008}: the rule picks the faster shape or
-        // stays within 4 % of it except for a few of the smallest problems.
-        const int units = (N + 31) / 32;
-        const int per_group = units >= 8 ? units / 8 : units;
-        const long cells_per_group = (long)((M + big::kRows - 1) / big::kRows) * per_group;
-        const bool duo = cells_per_group >= 256 && (K <= 1024 || per_group < 16);
-        if (!duo) return gemm_launch_big<big::Wide, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        return gemm_launch_big<big::Duo, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    }
+        return gemm_launch_large<OUT, false>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
@@ -1140,4 +1156,24 @@ extern "C" int quest_fused_matmul_dequantize_int4_int4t(void *mat_d, const uint8
                                      size_n, (hipStream_t)stream);
     return gemm_launch<OUT_FP16>(mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m, size_k, size_n,
                                  (hipStream_t)stream);
+}
+
+extern "C" int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                               const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                               const void *vec_a_mul, const void *vec_b_mul, int size_m,
+                                                               int size_k, int size_n, int dtype, void *stream) {
+    const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
+    if (rc != QUEST_OK) return rc;
+    if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (size_n & 7) return QUEST_ERR_BAD_SHAPE;                      // whole eights of weight rows: four gates, four ups
+    // only the large-tile kernel has this epilogue
+    if ((size_k & 127) != 0 || size_m <= 64 || (size_m & 1) != 0 || !aligned(vec_b_mul, 4) || !aligned(vec_a_mul, 4) ||
+        !aligned(mat_d, 8))
+        return QUEST_ERR_UNSUPPORTED;
+    if (dtype == QUEST_DTYPE_BF16)
+        return gemm_launch_large<OUT_BF16, true>(mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m,
+                                                 size_k, size_n, (hipStream_t)stream);
+    return gemm_launch_large<OUT_FP16, true>(mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m, size_k,
+                                             size_n, (hipStream_t)stream);
 }

@@ -195,15 +195,10 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
         v4u uq[8];
 #pragma unroll
         for (int s = 0; s < 8; s++) uq[s] = __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(ld_off + K * 2 + 32 * s), 0, 0);
-        auto silu = [](float g) { return __fdividef(g, 1.0f + __expf(-g)); };
 #pragma unroll
         for (int s = 0; s < 8; s++)
 #pragma unroll
-            for (int d = 0; d < 4; d++) {
-                const uint32_t a = pack2_rounded_products<DT>(silu(lo_f32<DT>(bq[s][d])), silu(hi_f32<DT>(bq[s][d])));
-                bq[s][d] = pack2_rounded_products<DT>(__fmul_rn(lo_f32<DT>(a), lo_f32<DT>(uq[s][d])),
-                                                      __fmul_rn(hi_f32<DT>(a), hi_f32<DT>(uq[s][d])));
-            }
+            for (int d = 0; d < 4; d++) bq[s][d] = silu_mul_pair<DT>(bq[s][d], uq[s][d]);
     }
     if constexpr (PRE != kPreNone) {
         if (pre_out != nullptr && live) {

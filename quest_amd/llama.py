@@ -97,6 +97,26 @@ class LlamaMLP(nn.Module):
         self.w2 = nn.Linear(config.n_embd, config.hidden_dim, bias=False)
         self.c_proj = nn.Linear(config.hidden_dim, config.n_embd, bias=False)
         self.w12 = None          # set by quantize_model(..., fuse_gate_up=True): one module for both
+        self.glu = None          # enable_swiglu_epilogue(): w12's packed rows in the order the gated-unit GEMM reads
+
+    def enable_swiglu_epilogue(self):
+        """A second copy of the fused gate/up weights with the rows interleaved in eights (four gate rows, then the four
+        up rows of the same outputs; `quest.swiglu_interleave_rows`), which lets the GEMM apply silu(gate) * up in
+        its epilogue.  Plain tensors, not buffers: they are derived data and stay out of checkpoints."""
+        w = self.w12
+        p = quest.swiglu_interleave_rows(w.w_int_packed.size(0) // 2, device=w.w_int_packed.device)
+        self.glu = (w.w_int_packed[p].contiguous(), w.w_scale[p].contiguous(), w.w_add[p].contiguous())
+
+    def swiglu_quantized(self, a_scale, a_int_packed, a_int_row_sum):
+        """silu(w1 x) * w2 x, (M, hidden), from the codes of x; the gated unit runs in the GEMM's epilogue when that
+        kernel takes the shape, otherwise in the torch expression on the plain GEMM's output."""
+        m = a_int_packed.size(0)
+        if self.glu is not None and m > 64 and m % 2 == 0 and a_int_packed.size(1) % 64 == 0 and self.w12.bias is None:
+            w_packed, w_scale, w_add = self.glu
+            return quest.fused_matmul_dequantize_swiglu_int4_int4t(a_int_packed, w_packed, a_int_row_sum, w_add, a_scale, w_scale)
+        gate_up = self.w12.forward_quantized(a_scale, a_int_packed, a_int_row_sum)
+        h = gate_up.size(-1) // 2
+        return F.silu(gate_up[..., :h]) * gate_up[..., h:]
 
     def forward(self, x):
         if self.w12 is not None:
@@ -174,8 +194,10 @@ class LlamaBlock(nn.Module):
             q = quest.add_rmsnorm_hadamard_quantize_int4(x2, branch.view(b * t, c), self.ln_1.weight, self.ln_1.eps)
         att = self.attn.attend(self.attn.c_attn.forward_quantized(*q).view(b, t, 3 * c), freqs_cis)
         q = quest.add_rmsnorm_hadamard_quantize_int4(x2, att.view(b * t, c), self.ln_2.weight, self.ln_2.eps)
-        gate_up = self.mlp.w12.forward_quantized(*q)
-        q = quest.silu_mul_hadamard_quantize_int4(gate_up)
+        if self.mlp.glu is not None:
+            q = quest.hadamard_quantize_int4(self.mlp.swiglu_quantized(*q))
+        else:
+            q = quest.silu_mul_hadamard_quantize_int4(self.mlp.w12.forward_quantized(*q))
         return x, self.mlp.c_proj.forward_quantized(*q).view(b, t, c)
 
 
@@ -241,7 +263,7 @@ def _pack(linear: nn.Linear, use_hadamard: bool, use_noop: bool) -> harness.Line
 
 @torch.no_grad()
 def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, fuse_gate_up: bool = True,
-                   fuse_producers: bool = False) -> Llama:
+                   fuse_producers: bool = False, swiglu_epilogue: bool = True) -> Llama:
     """bench_e2e.py:77-97 on an existing model: every linear under `transformer` becomes a `Linear4bit` holding the
     packed INT4 form of that linear's own weight ('int4'), or the same module in no-op mode ('noop'); 'bf16' leaves
     the dense linears.  The model must already sit on the GPU in bf16 or fp16."""
@@ -270,6 +292,8 @@ def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, 
         block.attn.fused_rope = bool(fuse_producers and not noop)
         block.fuse_producers = bool(fuse_producers and not noop and use_hadamard and fuse_gate_up and
                                     model.config.n_embd <= 4096 and model.config.hidden_dim <= 4096)
+        if block.fuse_producers and swiglu_epilogue and model.config.hidden_dim % 4 == 0:
+            mlp.enable_swiglu_epilogue()
     return model
 
 

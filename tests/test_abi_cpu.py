@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     names = declared_symbols()
     for n in ['quest_version', 'quest_status_string', 'quest_find_scale_int4', 'quest_quantize_int4',
-              'quest_add_mul_vv', 'quest_matmul_int4_int4t_int32', 'quest_fused_matmul_dequantize_int4_int4t',
+              'quest_add_mul_vv', 'quest_matmul_int4_int4t_int32', 'quest_fused_matmul_dequantize_int4_int4t', 'quest_fused_matmul_dequantize_swiglu_int4_int4t',
               'quest_hadamard128', 'quest_hadamard_quantize_int4', 'quest_hadamard_quantize_int4_rule',
               'quest_rmsnorm_hadamard_quantize_int4', 'quest_add_rmsnorm_hadamard_quantize_int4', 'quest_silu_mul_hadamard_quantize_int4', 'quest_rope_interleaved']:
         assert n in names

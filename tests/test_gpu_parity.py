@@ -188,6 +188,48 @@ def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
     assert ((got.double() - ref).norm() / ref.norm()) < 1e-2
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 768, 224), (66, 128, 8), (200, 256, 512), (300, 256, 1000), (16390, 256, 1000),
+                                   (16384, 128, 2048), (4096, 128, 4104)])
+def test_fused_matmul_dequantize_swiglu(quest, dtype, shape):
+    """The gate/up GEMM with silu(gate) * up in its epilogue = the plain fused GEMM on the same (interleaved) weight
+    rows followed by the activation kernel's own SwiGLU, bit for bit; and within 2 ulp of torch's CPU expression on the
+    plain GEMM's (bit-exact) output."""
+    m, k, n = shape                                            # n = 2 H weight rows
+    h = n // 2
+    g = torch.Generator().manual_seed(30)
+    a, b = rand_codes(m, k, 31), rand_codes(n, k, 32)          # b: gate rows 0..H-1, up rows H..2H-1
+    a_mul = (torch.rand(m, 1, generator=g) * 0.05 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g) * 0.05 + 0.01).to(dtype)
+    a_add = torch.randint(-200, 200, (m, 1), generator=g, dtype=torch.int32)
+    b_add = torch.randint(-200, 200, (n, 1), generator=g, dtype=torch.int32)
+    ga, gb, ga_add, gb_add, ga_mul, gb_mul = (t.to(DEV) for t in (a, b, a_add, b_add, a_mul, b_mul))
+    p = quest.swiglu_interleave_rows(h, device=DEV)
+    assert sorted(p.tolist()) == list(range(n)) and p[:8].tolist() == [0, 1, 2, 3, h, h + 1, h + 2, h + 3]
+    got = quest.fused_matmul_dequantize_swiglu_int4_int4t(ga, gb[p].contiguous(), ga_add, gb_add[p].contiguous(), ga_mul,
+                                                          gb_mul[p].contiguous())
+    assert got.shape == (m, h)
+    gate_up = quest.fused_matmul_dequantize_int4_int4t_bf16(ga, gb, ga_add, gb_add, ga_mul, gb_mul)     # (M, 2H), halves
+    if h % 128 == 0 and h <= 4096:
+        act = torch.empty(m, h, dtype=dtype, device=DEV)
+        quest.silu_mul_hadamard_quantize_int4(gate_up, x_act=act)
+        assert torch.equal(bits(got.cpu()), bits(act.cpu()))
+    cpu = gate_up.cpu()
+    want = torch.nn.functional.silu(cpu[:, :h]) * cpu[:, h:]
+    worst, frac = _ulp_stats(got.cpu(), want)
+    assert worst <= 2 and frac < 0.02, (worst, frac)
+
+
+def test_swiglu_gemm_refuses_small_batches(quest):
+    m, k, n = 16, 256, 64
+    a, b = rand_codes(m, k, 33).to(DEV), rand_codes(n, k, 34).to(DEV)
+    z = torch.zeros(m, 1, dtype=torch.int32, device=DEV)
+    zn = torch.zeros(n, 1, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError):
+        quest.fused_matmul_dequantize_swiglu_int4_int4t(a, b, z, zn, torch.ones(m, 1, dtype=torch.bfloat16, device=DEV),
+                                                        torch.ones(n, 1, dtype=torch.bfloat16, device=DEV))
+
+
 # --------------------------------------------------------------------------- H1 / H2
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('scale', [181. / 2048., 2. ** -3.5])
