@@ -142,7 +142,9 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                # enough cells for the two-workgroups-per-CU shape of the large-tile kernel (>= 256 cells of 256 tokens x
                # 32 channels per XCD group): few channels with a ragged last token tile; short K with a channel count
                # that takes the element-wise epilogue
-               (16390, 256, 1000), (4096, 128, 4100)]
+               (16390, 256, 1000), (4096, 128, 4100),
+               # the same with fewer than eight channel units (one scheduling group instead of one per XCD)
+               (65538, 128, 96)]
 
 
 @pytest.mark.parametrize('shape', GEMM_SHAPES)
