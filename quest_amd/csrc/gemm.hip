@@ -820,6 +820,16 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     // the lower half keeps group g and receives the upper half's part of it, the upper half does the same with
     // group g + 1), so that every lane stores 16 bytes = 8 consecutive channels and a half-wave pair covers 32
     // contiguous bytes of each token row; the four stores of a sub-tile complete its 64-byte row segments in L2.
+    if constexpr (OUT != OUT_INT32) {
+        // The tile's scale vectors were sent to LDS at its start; the stage synchronisations wait for them in passing
+        // (the counter runs in order and they are older than the tile's own stage loads) -- but only from the
+        // (kStages - 1)-th synchronisation on, the earlier ones leave the previous tile's stores and these loads in
+        // flight.  A K loop shorter than that (K <= 256, or 128 with three stages) has to wait here.
+        if (nk < C::kStages - 1) {
+            wait_vmcnt_imm<0>();
+            plain_barrier();
+        }
+    }
     constexpr int kEs = OUT == OUT_INT32 ? 4 : 2;                  // bytes per output element
     const bool fast = (N % (16 / kEs)) == 0;
     const bool interior = fast && tok0 + kRows <= M && ch0 + 32 * width <= N;
