@@ -171,7 +171,9 @@ def test_matmul_int32_extreme_codes(quest):
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768, 224), (16, 4096, 4096), (1, 11008, 4096), (257, 256, 301),
                                    (8, 4096, 11008), (3, 384, 18), (33, 1152, 62), (64, 640, 100), (20, 2304, 47),
-                                   (16390, 256, 1000), (4096, 128, 4100)])
+                                   (16390, 256, 1000), (4096, 128, 4100),
+                                   # one or two pipeline stages per tile: the epilogue must wait for its scale vectors itself
+                                   (4096, 256, 2048), (16384, 128, 2048)])
 def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
     m, k, n = shape
     g = torch.Generator().manual_seed(6)
