@@ -333,6 +333,29 @@ def bench_forward(dev):
             'wiring': 'QKV fused (as the reference); gate and up share one quantisation and one GEMM'}
 
 
+def bench_small_layer_gpu(quest, dev):
+    """The CPU baseline's workload (fp16 [512,1024] x [1024,1024]^T, Hadamard on, absmax-scaled weights) through the
+    HIP path, as a replayed HIP graph of 100 layers: the figure to set beside `cpu_baseline`."""
+    from quest_amd import harness
+    torch.manual_seed(0)
+    m, k, n = 512, 1024, 1024
+    x = torch.randn(m, k).half().to(dev)
+    w = (torch.randn(n, k) * 0.02).half().to(dev)
+    wp, ws, wa, _ = harness.preprocess_weight(w, use_hadamard=True, w_scale_mode='absmax')
+    scale = torch.empty(m, 1, dtype=x.dtype, device=dev)
+    packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+    row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
+    out = torch.empty(m, n, dtype=x.dtype, device=dev)
+
+    def layer(_):
+        quest.hadamard_quantize_int4(x, scale, packed, row_sum)
+        quest.fused_matmul_dequantize_int4_int4t_bf16(packed, wp, row_sum, wa, scale, ws, out)
+
+    ms = launches_ms(layer, 100, 10)
+    return {'ms_per_call': ms, 'value': 2.0 * m * n * k / (ms * 1e-3) / 1e12, 'unit': 'TOPS',
+            'what': 'the same layer through the HIP path on the GPU (graph replay, median of seven)'}
+
+
 def bench_cpu_baseline():
     """The CPU oracle on the reference's CPU-runnable case: fp16 [512,1024] x [1024,1024]^T, Hadamard
     as F.linear, scale, quantise, integer GEMM through fp64 as the reference's own check does, and
@@ -410,6 +433,8 @@ def main():
     fwd = None if args.no_forward else bench_forward(dev)
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
+    if cpu is not None:
+        cpu['gpu_same_workload'] = bench_small_layer_gpu(quest, dev)
 
     roofline = {'bound': 'mfma', 'achieved': lin['gemm_tops'], 'peak': INT8_MFMA_PEAK_TOPS, 'unit': 'TOP/s',
                 'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES,
