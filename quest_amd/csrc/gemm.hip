@@ -631,6 +631,7 @@ __device__ __forceinline__ void wait_stage(int extra) {
         case 28: wait_vmcnt_imm<kBase + 28>(); break;
         case 20: wait_vmcnt_imm<kBase + 20>(); break;
         case 12: wait_vmcnt_imm<kBase + 12>(); break;
+        case 8: wait_vmcnt_imm<kBase + 8>(); break;
         case 4: wait_vmcnt_imm<kBase + 4>(); break;
         default: wait_vmcnt_imm<kBase>(); break;
     }
@@ -666,11 +667,12 @@ struct Frags {
 //   * `sync` runs after slot kSyncSlot (-1: none) and the stage's loads, dma(0..kLoads), follow one per few slots;
 //   * NEXT: the packed fragments of the next k-pair are read from LDS in the slots after that, up to 3/8 of the
 //     way, and split into `nxt` (3 VALU ops per dword) over the second half of the slots.
-template <typename C, int NA, bool NEXT, int kSyncSlot, typename Sync, typename Dma>
+// TB = token sub-tiles of 32 the wave multiplies (4, or 2 when all four waves split the tokens of a narrow tile).
+template <typename C, int NA, int TB, bool NEXT, int kSyncSlot, typename Sync, typename Dma>
 __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Frags &cur, Frags &nxt, const uint8_t *rd_tok,
                                        const uint8_t *rd_chn, Sync &&sync, Dma &&dma) {
-    constexpr int S = 8 * NA;                 // slots
-    constexpr int F = 4 + NA;                 // fragments per k-pair
+    constexpr int S = 2 * TB * NA;            // slots
+    constexpr int F = TB + NA;                // fragments per k-pair
     constexpr int V = F * 4;                  // dwords to split
     constexpr int R0 = kSyncSlot + 1;         // reads go into slots [R0, R1)
     constexpr int R1 = S * 3 / 8 > R0 ? S * 3 / 8 : R0 + 1;
@@ -678,7 +680,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
     v4i raw[8];
 #pragma unroll
     for (int i = 0; i < S; i++) {
-        const int a = i >> 3, odd = (i >> 2) & 1, b = i & 3;
+        const int a = i / (2 * TB), odd = (i / TB) & 1, b = i % TB;
         acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(odd ? cur.co[a] : cur.ce[a], odd ? cur.to[b] : cur.te[b], acc[a][b],
                                                           0, 0, 0);
         if (i == kSyncSlot) sync();
@@ -693,7 +695,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
             if (i >= R0 && i < R1) {
 #pragma unroll
                 for (int r = (i - R0) * F / (R1 - R0); r < (i - R0 + 1) * F / (R1 - R0); r++)
-                    raw[r] = *reinterpret_cast<const v4i *>(r < 4 ? rd_tok + r * 32 * kRowB : rd_chn + (r - 4) * 32 * kRowB);
+                    raw[r] = *reinterpret_cast<const v4i *>(r < TB ? rd_tok + r * 32 * kRowB : rd_chn + (r - TB) * 32 * kRowB);
             }
             if (i >= U0) {
 #pragma unroll
@@ -701,7 +703,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
                     const int f = v >> 2, d = v & 3;
                     const uint32_t pk = (uint32_t)raw[f][d];
                     const int ev = (int)((pk << 4) & 0xF0F0F0F0u), od = (int)(pk & 0xF0F0F0F0u);
-                    if (f < 4) { nxt.te[f][d] = ev; nxt.to[f][d] = od; } else { nxt.ce[f - 4][d] = ev; nxt.co[f - 4][d] = od; }
+                    if (f < TB) { nxt.te[f][d] = ev; nxt.to[f][d] = od; } else { nxt.ce[f - TB][d] = ev; nxt.co[f - TB][d] = od; }
                 }
             }
         }
@@ -709,7 +711,7 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
     }
 }
 
-template <typename C, int OUT, bool GLU, int NA>
+template <typename C, int OUT, bool GLU, int NA, int TB>
 __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, const int32_t *__restrict__ a_add,
                                          const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
                                          const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0,
@@ -721,13 +723,15 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     // peaks, and a scratch reload waits on the vector-memory counter, i.e. on every store and load in flight.
     const int lane = fresh_lane_id();
     const int wave = ldr.wave;                                      // scalar
-    const int wt = wave >> 1;
+    // the wave's token rows inside the tile: a half of 128 (the other wave of the half takes the other channel units),
+    // or, in a tile of one or two channel units, a quarter of 64 with all of the tile's units
+    const int tok_in_tile = TB == 4 ? (wave >> 1) * 128 : wave * 64;
     const int li = lane & 31;
     const int lg = lane >> 5;
     const int nk = K / 128;
 
     // operand reads: row li of a 32-row sub-tile; the 16-byte chunk 2 j + lg of its 64-byte stage row (k-pair j)
-    const int rd_t = (wt * 128 + li) * kRowB;
+    const int rd_t = (tok_in_tile + li) * kRowB;
     const int rd_c = kTileB + (unit0 * 32 + li) * kRowB;
     int rd_j[2];
 #pragma unroll
@@ -737,7 +741,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
 #pragma unroll
     for (int a = 0; a < NA; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++)
+        for (int b = 0; b < TB; b++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
 
@@ -793,23 +797,23 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             const int slot = pp.it % C::kStages;
             const uint8_t *t0 = tok_base(slot, 0), *c0 = chn_base(slot, 0);
 #pragma unroll
-            for (int f = 0; f < 4 + NA; f++) {
-                const v4i raw = *reinterpret_cast<const v4i *>(f < 4 ? t0 + f * 32 * kRowB : c0 + (f - 4) * 32 * kRowB);
+            for (int f = 0; f < TB + NA; f++) {
+                const v4i raw = *reinterpret_cast<const v4i *>(f < TB ? t0 + f * 32 * kRowB : c0 + (f - TB) * 32 * kRowB);
                 v4i ev, od;
                 split16(raw, ev, od);
-                if (f < 4) { u0.te[f] = ev; u0.to[f] = od; } else { u0.ce[f - 4] = ev; u0.co[f - 4] = od; }
+                if (f < TB) { u0.te[f] = ev; u0.to[f] = od; } else { u0.ce[f - TB] = ev; u0.co[f - TB] = od; }
             }
         }
         for (int kt = 0; kt < nk - 1; kt++) {
             const int slot = pp.it % C::kStages, next = (pp.it + 1) % C::kStages;
-            k_pair<C, NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
-            k_pair<C, NA, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync, dma);
+            k_pair<C, NA, TB, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
+            k_pair<C, NA, TB, true, -1>(acc, u1, u0, tok_base(next, 0), chn_base(next, 0), no_sync, dma);
             pp.it++;
         }
         {   // last stage of the tile: nothing of the next tile is read here (its channel rows sit elsewhere)
             const int slot = pp.it % C::kStages;
-            k_pair<C, NA, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
-            k_pair<C, NA, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync, dma);
+            k_pair<C, NA, TB, true, 1>(acc, u0, u1, tok_base(slot, 1), chn_base(slot, 1), sync, dma);
+            k_pair<C, NA, TB, false, -1>(acc, u1, u0, nullptr, nullptr, no_sync, dma);
             pp.it++;
         }
     }
@@ -838,23 +842,24 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     const int lane_e = fresh_lane_id();
     const int li_e = lane_e & 31;
     const int lg_e = lane_e >> 5;
+    const int tok_e = TB == 4 ? (wave >> 1) * 128 : wave * 64;      // from the scalar wave number: nothing kept alive
     if (NA > 0 && fast) {
         int t_add[4];                                              // of the tokens whose values this lane converts
         float t_half_mul[4];
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
+        for (int b = 0; b < TB; b++) {
             t_add[b] = 0;
             t_half_mul[b] = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                t_add[b] = w_add[wt * 128 + b * 32 + li_e];
-                t_half_mul[b] = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
+                t_add[b] = w_add[tok_e + b * 32 + li_e];
+                t_half_mul[b] = __fmul_rn(0.5f, to_f32<DT>(w_mul[tok_e + b * 32 + li_e]));
             }
         }
         // GLU: the output has N / 2 columns, 16 per channel unit (see the store below)
         constexpr int kOutPerUnit = GLU ? 16 : 32;
         const int n_out = GLU ? N >> 1 : N;
         uint8_t *out_lane = reinterpret_cast<uint8_t *>(out) +
-                            ((size_t)(tok0 + wt * 128 + li_e) * n_out + (size_t)((ch0 >> 5) + unit0) * kOutPerUnit) * kEs;
+                            ((size_t)(tok0 + tok_e + li_e) * n_out + (size_t)((ch0 >> 5) + unit0) * kOutPerUnit) * kEs;
         // Loop order.  One workgroup per CU: channel unit outside, so that a unit's 32 scale values are read from
         // LDS once.  Two per CU: token sub-tile outside, so that the stores of consecutive iterations complete whole
         // 128-byte lines of the same rows (measured -3..-6 % run time at short K; nothing for the wide shape).
@@ -862,9 +867,9 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         int adds[16];
         float muls[16];
 #pragma unroll
-        for (int o = 0; o < (kTokOuter ? 4 : NA); o++) {
+        for (int o = 0; o < (kTokOuter ? TB : NA); o++) {
 #pragma unroll
-          for (int i = 0; i < (kTokOuter ? NA : 4); i++) {
+          for (int i = 0; i < (kTokOuter ? NA : TB); i++) {
             const int a = kTokOuter ? i : o, b = kTokOuter ? o : i;
             if constexpr (OUT != OUT_INT32) {
               if (kTokOuter || i == 0) {
@@ -880,7 +885,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
               }
             }
             {
-                const bool tok_ok = tok0 + wt * 128 + b * 32 + li_e < M;
+                const bool tok_ok = tok0 + tok_e + b * 32 + li_e < M;
                 uint8_t *dst = out_lane + ((size_t)b * 32 * n_out + a * kOutPerUnit) * kEs;
                 if constexpr (OUT == OUT_INT32) {
 #pragma unroll
@@ -930,14 +935,14 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     } else if (NA > 0 && !GLU) {
         // generic path (N not a multiple of 8 / 4): element-wise stores straight from the accumulators
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const int tok = tok0 + wt * 128 + b * 32 + li_e;
+        for (int b = 0; b < TB; b++) {
+            const int tok = tok0 + tok_e + b * 32 + li_e;
             if (tok >= M) continue;
             int t_add = 0;
             float t_half_mul = 0.f;
             if constexpr (OUT != OUT_INT32) {
-                t_add = w_add[wt * 128 + b * 32 + li_e];
-                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[wt * 128 + b * 32 + li_e]));
+                t_add = w_add[tok_e + b * 32 + li_e];
+                t_half_mul = __fmul_rn(0.5f, to_f32<DT>(w_mul[tok_e + b * 32 + li_e]));
             }
 #pragma unroll
             for (int a = 0; a < NA; a++) {
@@ -966,7 +971,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     // store instruction of the fast path was issued with all its lanes (an interior tile), otherwise none
     // (the next tile's four vector loads, issued right after this point, are always exact)
     if constexpr (OUT != OUT_INT32) {
-        pp.store_extra = (interior ? 8 * NA : 0) + 4;
+        pp.store_extra = (interior ? 2 * TB * NA : 0) + 4;
         pp.store_syncs = C::kStages - 2;
     } else {
         pp.store_extra = 0;
@@ -1043,8 +1048,15 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
 #define QUEST_BIG_TILE(NA) \
-    big_tile<C, OUT, GLU, NA>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
-        if constexpr (C::kMaxUnits > 4) {
+    big_tile<C, OUT, GLU, NA, 4>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
+        if (cc.width <= 2) {
+            // a tile of one or two channel units (small problems, the ends of runs): every wave takes a quarter of the
+            // tokens and all of the units, instead of two of the four waves idling or holding half-empty accumulators
+            if (cc.width == 2)
+                big_tile<C, OUT, GLU, 2, 2>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, 0, 2);
+            else
+                big_tile<C, OUT, GLU, 1, 2>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, 0, 1);
+        } else if constexpr (C::kMaxUnits > 4) {
             switch (na) {
                 case 4: QUEST_BIG_TILE(4); break;
                 case 3: QUEST_BIG_TILE(3); break;
