@@ -1142,7 +1142,9 @@ template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
     // a handful of tokens: the weight-streaming kernel
-    if (M <= 64) {
+    // (up to 64 of them always; up to 128 while its N / 16 workgroups still run as one round, where it is twice as
+    // fast as large tiles that would be half empty)
+    if (M <= 64 || (M <= 128 && N <= 8192)) {
         const int rc = launch_gemm_decode(OUT, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
         if (rc != QUEST_ERR_UNSUPPORTED) return rc;
     }

@@ -1,4 +1,4 @@
-// Packed-INT4 x packed-INT4 GEMM for a handful of tokens (M <= 64): the weight matrix is streamed
+// Packed-INT4 x packed-INT4 GEMM for a handful of tokens (M <= 128): the weight matrix is streamed
 // from HBM exactly once and that stream is the whole cost, so the kernel is laid out around it.
 //
 // Same arithmetic and outputs as the large GEMM (gemm-quest/quest/matmul_kernel.cu:8-63 and
@@ -41,7 +41,7 @@ __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
 
 // TM = token tiles of 16 (M <= 16 TM)
 template <int OUT, int TM>
-__global__ void __launch_bounds__(64 * kWaves, TM == 1 ? 8 : TM == 2 ? 4 : 2)
+__global__ void __launch_bounds__(64 * kWaves, TM == 1 ? 8 : TM == 2 ? 4 : TM == 4 ? 2 : 1)
 gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                         const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
                         const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul, int M, int N, int K) {
@@ -183,16 +183,17 @@ static int launch_out(void *out, const uint8_t *a, const uint8_t *b, const int32
                       const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
     if (M <= 16) launch_tm<OUT, 1>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     else if (M <= 32) launch_tm<OUT, 2>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    else launch_tm<OUT, 4>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    else if (M <= 64) launch_tm<OUT, 4>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    else launch_tm<OUT, 8>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return launch_status();
 }
 
 }  // namespace decode
 
-// The weight-streaming kernel applies to M <= 64 and K a multiple of 128 (whole 64-byte pieces); QUEST_ERR_UNSUPPORTED otherwise.
+// The weight-streaming kernel applies to M <= 128 and K a multiple of 128 (whole 64-byte pieces); QUEST_ERR_UNSUPPORTED otherwise.
 int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                        const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    if (M > 64 || (K & 127) != 0 || !aligned(a, 16) || !aligned(b, 16)) return QUEST_ERR_UNSUPPORTED;
+    if (M > 128 || (K & 127) != 0 || !aligned(a, 16) || !aligned(b, 16)) return QUEST_ERR_UNSUPPORTED;
     switch (out_kind) {
         case OUT_BF16: return decode::launch_out<OUT_BF16>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
         case OUT_FP16: return decode::launch_out<OUT_FP16>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);

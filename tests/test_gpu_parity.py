@@ -138,7 +138,7 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                (33, 96, 7), (512, 1024, 1024), (300, 160, 257), (256, 2048, 256),
                # a handful of tokens (the weight-streaming kernel): 64-byte row tails, ragged N, each token-tile count
                (3, 384, 18), (16, 128, 16), (17, 1152, 64), (32, 640, 100), (40, 2304, 47), (64, 8192, 32), (5, 28672, 24),
-               (12, 160, 40),
+               (12, 160, 40), (65, 256, 48), (100, 1152, 300), (128, 4096, 512), (127, 384, 33),
                # enough cells for the two-workgroups-per-CU shape of the large-tile kernel (>= 256 cells of 256 tokens x
                # 32 channels per XCD group): few channels with a ragged last token tile; short K with a channel count
                # that takes the element-wise epilogue
@@ -171,6 +171,7 @@ def test_matmul_int32_extreme_codes(quest):
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768, 224), (16, 4096, 4096), (1, 11008, 4096), (257, 256, 301),
                                    (8, 4096, 11008), (3, 384, 18), (33, 1152, 62), (64, 640, 100), (20, 2304, 47),
+                                   (65, 256, 48), (100, 1152, 300), (128, 4096, 512),
                                    (16390, 256, 1000), (4096, 128, 4100),
                                    # one or two pipeline stages per tile: the epilogue must wait for its scale vectors itself
                                    (4096, 256, 2048), (16384, 128, 2048)])
