@@ -38,10 +38,10 @@ LAST = {'min_ms': None}      # fastest replay of the most recent launches_ms() c
 INT8_MFMA_PEAK_TOPS = 5000.0
 
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
-# scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.99982, WRITE_SIZE x 1.0);
+# scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
-TRAFFIC_GEMM_BYTES = 344317277
-TRAFFIC_QUANTIZE_BYTES = 84106458
+TRAFFIC_GEMM_BYTES = 344181278
+TRAFFIC_QUANTIZE_BYTES = 84105486
 
 
 def event_pairs(n):
