@@ -194,6 +194,18 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         return gemm
 
     gemm_quantized_ms = launches_ms(gemm_launcher(a_packed, a_row_sum, a_scale), max(steps, 100))
+    # the same with the weights rotated through 14 copies (315 MB, more than the Infinity Cache holds), as a model
+    # with many layers would stream them from HBM
+    w_copies = [w_packed] + [w_packed.clone() for _ in range(13)]
+    u_args = (_lib.ptr(u_row_sum), _lib.ptr(w_add), _lib.ptr(u_scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype])
+    w_ptrs = [_lib.ptr(w) for w in w_copies]
+
+    def gemm_rotating(i):
+        if lib.quest_fused_matmul_dequantize_int4_int4t(_lib.ptr(out), _lib.ptr(u_packed), w_ptrs[i % 14], *u_args, current_stream()) != 0:
+            raise RuntimeError('GEMM launch failed')
+
+    gemm_rotating_ms = launches_ms(gemm_rotating, 98)
+    del w_copies
     gemm_ms = launches_ms(gemm_launcher(u_packed, u_row_sum, u_scale), max(steps, 100))
     gemm_min_ms = LAST['min_ms']
     ops = 2.0 * m * n * k
@@ -207,6 +219,7 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         'gemm_tops': ops / (gemm_ms * 1e-3) / 1e12,
         'gemm_in_step_ms': gemm_in_step_ms,
         'gemm_quantized_acts_ms': gemm_quantized_ms,
+        'gemm_rotating_weights_ms': gemm_rotating_ms,
         'quant_ms': quant_ms,
     }
 
@@ -440,6 +453,7 @@ def main():
                 'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES,
                 'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
                 'us_per_launch_min': lin['gemm_min_ms'] * 1e3,
+                'us_per_launch_weights_from_hbm': lin['gemm_rotating_weights_ms'] * 1e3,
                 'algorithmic_ops': 2.0 * 4096 * 4096 * 11008,
                 'workload': 'uniform random INT4 codes on both sides, M=4096 K=4096 N=11008, fp16 out'}
     line = {
