@@ -1079,6 +1079,192 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
 
 }  // namespace big
 
+// =================================================================================================
+// Small-tile kernel (K % 256 == 0): a few hundred tokens
+// =================================================================================================
+// Between the weight-streaming kernel (a handful of tokens) and the large tiles (thousands) there are too few
+// 256-token tiles to fill the chip, and a large tile that is one or two channel units wide leaves a lone wave per
+// SIMD issuing a few hundred instructions per stage around four multiplications.  Here a workgroup of eight waves
+// owns 64 tokens x 64 channels: waves 0-3 and 4-7 each hold the four 32 x 32 quadrants and split K between them
+// (the first and the second k-pair of every 128-k sub-stage; summed through LDS at the end), which gives every SIMD
+// two waves of a tile and, with two or more tiles per CU, four or more.  Operands travel as in the large-tile
+// kernel: packed bytes HBM -> LDS by direct loads (stages of 256 k = two sub-stages of 64-byte rows, each wave
+// bringing 16 token or channel rows), 16 packed bytes per lane per k-pair, split into the int8 vectors of
+// 16 * even-k and 16 * odd-k nibbles for two MFMA k-steps.
+namespace small {
+
+constexpr int kTok = 64, kChn = 64;
+constexpr int kRowB = 64;                         // packed bytes per row per sub-stage (128 k)
+constexpr int kHalfB = (kTok + kChn) * kRowB;     // 8 KiB: the token rows of a sub-stage, then its channel rows
+constexpr int kStageB = 2 * kHalfB;               // 16 KiB: 256 k
+constexpr int kStages = 4;
+constexpr int kLdsB = kStages * kStageB;          // 64 KiB: two workgroups per CU
+
+template <int OUT, bool GLU>
+__global__ void __launch_bounds__(512, 4)
+gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
+                       const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
+                       const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
+                       int M, int N, int K, int tiles_t, int tiles_c) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsB];
+    constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int lane = (int)threadIdx.x & 63;
+    // Workgroups are dealt to the eight XCDs in turn: all token tiles of a channel tile go to one XCD, whose L2 then
+    // fetches those weight rows once.  The grid is rounded up to whole eights of channel tiles.
+    const int xcd = (int)blockIdx.x & 7, local = (int)blockIdx.x >> 3;
+    const int ct = (local / tiles_t) * 8 + xcd;
+    const int tt = local % tiles_t;
+    if (ct >= tiles_c) return;                                   // uniform: the whole workgroup
+    const int tok0 = tt * kTok, ch0 = ct * kChn;
+    const int kbytes = K >> 1;
+    const int nk = K / 256;
+
+    // ---- loads: waves 0-3 bring token rows [16 w, +16), waves 4-7 channel rows [16 (w - 4), +16) of each sub-stage
+    const bool ld_tok = wave < 4;
+    const __amdgpu_buffer_rsrc_t src = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(ld_tok ? act : wgt), 0, (ld_tok ? M : N) * kbytes, 0x00020000);      // rows past the end read as zeros
+    // lane p covers row p / 4 of the 16; LDS slot p (lane order) must hold chunk (p & 3) ^ ((row >> 2) & 3) of that row
+    const uint32_t voff = (uint32_t)((ld_tok ? tok0 : ch0) + (wave & 3) * 16 + (lane >> 2)) * (uint32_t)kbytes +
+                          (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+    uint8_t *const dst0 = lds + (ld_tok ? 0 : kTok * kRowB) + (wave & 3) * 16 * kRowB;
+    auto issue = [&](int kt, int slot) {
+        uint8_t *d = dst0 + slot * kStageB;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (__attribute__((address_space(3))) void *)d, 16, voff, kt * 128, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (__attribute__((address_space(3))) void *)(d + kHalfB), 16, voff,
+                                                 kt * 128 + 64, 0, 0);
+    };
+
+    // ---- operand reads: row li of the wave's 32 token / channel rows, 16-byte chunk 2 kh + lg of the 64-byte row
+    const int kh = wave >> 2, tr = (wave >> 1) & 1, tc = wave & 1;
+    const int li = lane & 31, lg = lane >> 5;
+    const int rd_x = ((2 * kh + lg) ^ ((li >> 2) & 3)) * 16;
+    const int rd_t = (tr * 32 + li) * kRowB + rd_x;
+    const int rd_c = (kTok + tc * 32 + li) * kRowB + rd_x;
+
+    v16i acc, acc1;                                      // one per sub-stage: two independent chains of MFMAs
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = acc1[r] = 0;
+
+    // Stages 0 .. kStages - 2 in flight before the loop; past the end of K the last stage is fetched again (into a
+    // free slot), which keeps the count of outstanding loads uniform.
+#pragma unroll
+    for (int s = 0; s < kStages - 1; s++) issue(s < nk ? s : nk - 1, s);
+    for (int kt = 0; kt < nk; kt++) {
+        big::wait_vmcnt_imm<2 * (kStages - 2)>();        // this wave's share of stage kt has landed ...
+        big::plain_barrier();                            // ... and everyone else's; the slot of stage kt - 1 is free
+        const int nx = kt + kStages - 1;
+        issue(nx < nk ? nx : nk - 1, nx % kStages);
+        const uint8_t *sb = lds + (kt % kStages) * kStageB;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const v4i rt = *reinterpret_cast<const v4i *>(sb + h * kHalfB + rd_t);
+            const v4i rc = *reinterpret_cast<const v4i *>(sb + h * kHalfB + rd_c);
+            v4i te, to, ce, co;
+            big::split16(rt, te, to);
+            big::split16(rc, ce, co);
+            if (h == 0) {
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to, acc, 0, 0, 0);
+            } else {
+                acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te, acc1, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to, acc1, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] += acc1[r];
+    big::wait_vmcnt_imm<0>();                            // no direct-to-LDS load may still be writing ...
+    big::plain_barrier();                                // ... and nobody still reading when the stages are reused
+
+    // ---- the two K halves: waves 4-7 park their accumulators in LDS, waves 0-3 add them and finish the tile
+    int32_t *red = reinterpret_cast<int32_t *>(lds);     // 4 waves x 16 registers x 64 lanes: 16 KiB
+    if (kh == 1) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[((wave & 3) * 16 + r) * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] += red[(wave * 16 + r) * 64 + lane];
+
+    // ---- epilogue: accumulator register r of lane (li, lg) is 256 x the product for token li and channel
+    // 8 (r / 4) + 4 lg + r % 4 of the wave's quadrant
+    const int tok = tok0 + tr * 32 + li;
+    const int cb = ch0 + tc * 32;
+    const bool tok_ok = tok < M;
+    if constexpr (OUT == OUT_INT32) {
+        int32_t *dst = reinterpret_cast<int32_t *>(out) + (size_t)(tok_ok ? tok : 0) * N;
+        const bool vec_ok = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;     // 16-byte stores
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+            const int c = cb + rg * 8 + lg * 4;
+            if (!tok_ok) continue;
+            if (vec_ok) {
+                if (c < N)
+                    *reinterpret_cast<int4 *>(dst + c) =
+                        make_int4(acc[rg * 4] >> 8, acc[rg * 4 + 1] >> 8, acc[rg * 4 + 2] >> 8, acc[rg * 4 + 3] >> 8);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (c + e < N) dst[c + e] = acc[rg * 4 + e] >> 8;
+            }
+        }
+    } else {
+        const int t_add = tok_ok ? a_add[tok] : 0;
+        const float t_half_mul = tok_ok ? __fmul_rn(0.5f, to_f32<DT>(a_mul[tok])) : 0.f;
+        // GLU: weight rows interleaved in eights, the output has N / 2 columns (the caller guarantees N % 8 == 0 and
+        // an 8-byte aligned output)
+        uint16_t *dst = reinterpret_cast<uint16_t *>(out) + (size_t)(tok_ok ? tok : 0) * (GLU ? N >> 1 : N);
+        const bool fast = GLU || ((N & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0);     // 16-byte stores
+        float v[4][4];
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int c = cb + rg * 8 + lg * 4 + e;
+                const int cc = c < N ? c : N - 1;
+                // the accumulator is 256 C exactly, so 2 C is one arithmetic shift
+                const float lhs = (float)((acc[rg * 4 + e] >> 7) + t_add + b_add[cc]);
+                const float rhs = __fmul_rn(t_half_mul, to_f32<DT>(b_mul[cc]));
+                v[rg][e] = __fmul_rn(lhs, rhs);
+            }
+        }
+        if (fast) {
+            // the half-waves trade register groups, so that every lane stores 16 bytes = 8 consecutive channels
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++) {
+                const uint32_t x00 = pack2_rounded_products<DT>(v[2 * pr][0], v[2 * pr][1]);
+                const uint32_t x01 = pack2_rounded_products<DT>(v[2 * pr][2], v[2 * pr][3]);
+                const uint32_t x10 = pack2_rounded_products<DT>(v[2 * pr + 1][0], v[2 * pr + 1][1]);
+                const uint32_t x11 = pack2_rounded_products<DT>(v[2 * pr + 1][2], v[2 * pr + 1][3]);
+                // lower half-wave: group 2 pr complete; upper half-wave: group 2 pr + 1 complete
+                const auto s0 = __builtin_amdgcn_permlane32_swap(x00, x10, false, false);
+                const auto s1 = __builtin_amdgcn_permlane32_swap(x01, x11, false, false);
+                const int c = cb + (2 * pr + lg) * 8;
+                if constexpr (GLU) {
+                    // the lane holds four gate rows, then the four up rows of the same outputs
+                    if (tok_ok && c < N)
+                        *reinterpret_cast<uint2 *>(dst + (c >> 1)) =
+                            make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
+                } else if (tok_ok && c < N) {
+                    *reinterpret_cast<uint4 *>(dst + c) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                }
+            }
+        } else if (!GLU && tok_ok) {
+#pragma unroll
+            for (int rg = 0; rg < 4; rg++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int c = cb + rg * 8 + lg * 4 + e;
+                    if (c < N) dst[c] = (uint16_t)from_f32<DT>(v[rg][e]);
+                }
+        }
+    }
+}
+
+}  // namespace small
+
 static int device_cu_count() {
     static int cus = 0;
     if (cus == 0) {
@@ -1121,6 +1307,27 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
     return launch_status();
 }
 
+// A few hundred tokens: small tiles, while there are at most four of them per CU (beyond that the large tiles' operand
+// reuse wins), or eight where M would leave the last 256-token tile mostly empty.  Measured against the other kernels
+// over M from 65 to 2048 with (K, N) from (1024, 3072) to (8192, 8192): 1.2 to 2.6 x faster where this picks it.
+static bool small_tiles_pay(int M, int K, int N) {
+    if ((K & 255) != 0 || M <= 64) return false;
+    const long tiles = (long)((M + small::kTok - 1) / small::kTok) * ((N + small::kChn - 1) / small::kChn);
+    const long per_cu = (tiles + device_cu_count() - 1) / device_cu_count();
+    return per_cu <= 4 || (per_cu <= 8 && M < 1024 && (M & 255) != 0);
+}
+
+template <int OUT, bool GLU = false>
+static int gemm_launch_small(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
+                             const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    const int tiles_t = (M + small::kTok - 1) / small::kTok;
+    const int tiles_c = (N + small::kChn - 1) / small::kChn;
+    const long grid = (long)tiles_t * ((tiles_c + 7) / 8) * 8;
+    small::gemm_w4a4_small_kernel<OUT, GLU><<<dim3((unsigned)grid), dim3(512), 0, st>>>(
+        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, tiles_t, tiles_c);
+    return launch_status();
+}
+
 // Wide (256 x 256 tiles, a lone wave per SIMD) has the cheaper main loop; Duo (256 x 128, two workgroups per CU)
 // hides epilogues and waits.  Duo wins where there is enough work for full-width tiles on 512 workgroups (256 cells
 // of 256 tokens x 32 channels per XCD group) and the epilogue weighs much: K short, or fewer than 16 channel units
@@ -1130,6 +1337,7 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 template <int OUT, bool GLU>
 static int gemm_launch_large(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                              const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    if (small_tiles_pay(M, K, N)) return gemm_launch_small<OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     const int units = (N + 31) / 32;
     const int per_group = units >= 8 ? units / 8 : units;
     const long cells_per_group = (long)((M + big::kRows - 1) / big::kRows) * per_group;
@@ -1143,9 +1351,10 @@ static int gemm_launch_large(void *out, const uint8_t *a, const uint8_t *b, cons
 template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+    if (small_tiles_pay(M, K, N)) return gemm_launch_small<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     // a handful of tokens: the weight-streaming kernel
-    // (up to 64 of them always; up to 128 while its N / 16 workgroups still run as one round, where it is twice as
-    // fast as large tiles that would be half empty)
+    // (up to 64 of them always; where K rules out the small tiles, up to 128 while its N / 16 workgroups still run
+    // as one round: twice as fast as large tiles that would be half empty)
     if (M <= 64 || (M <= 128 && N <= 8192)) {
         const int rc = launch_gemm_decode(OUT, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
         if (rc != QUEST_ERR_UNSUPPORTED) return rc;

@@ -144,7 +144,13 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                # that takes the element-wise epilogue
                (16390, 256, 1000), (4096, 128, 4100),
                # the same with fewer than eight channel units (one scheduling group instead of one per XCD)
-               (65538, 128, 96)]
+               (65538, 128, 96),
+               # a few hundred tokens with K % 256 == 0 (the small-tile kernel): ragged token and channel tiles, channel
+               # counts that take the element-wise epilogue, one and several tiles per CU, a single 256-k stage
+               (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048), (66, 4096, 8),
+               (640, 2816, 1024),
+               # the same token counts with K % 256 != 0 (large tiles one or two channel units wide)
+               (200, 384, 512), (300, 640, 1000)]
 
 
 @pytest.mark.parametrize('shape', GEMM_SHAPES)
@@ -174,7 +180,12 @@ def test_matmul_int32_extreme_codes(quest):
                                    (65, 256, 48), (100, 1152, 300), (128, 4096, 512),
                                    (16390, 256, 1000), (4096, 128, 4100),
                                    # one or two pipeline stages per tile: the epilogue must wait for its scale vectors itself
-                                   (4096, 256, 2048), (16384, 128, 2048)])
+                                   (4096, 256, 2048), (16384, 128, 2048),
+                                   # a few hundred tokens, K % 256 == 0 (small tiles): ragged tiles, vector and element-wise stores
+                                   (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048),
+                                   (66, 4096, 8), (640, 2816, 1024),
+                                   # ... and K % 256 != 0 (narrow large tiles)
+                                   (200, 384, 512), (300, 640, 1000)])
 def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
     m, k, n = shape
     g = torch.Generator().manual_seed(6)
@@ -195,7 +206,8 @@ def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
 
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768, 224), (66, 128, 8), (200, 256, 512), (300, 256, 1000), (16390, 256, 1000),
-                                   (16384, 128, 2048), (4096, 128, 4104)])
+                                   (16384, 128, 2048), (4096, 128, 4104), (200, 384, 512), (130, 1024, 4104),
+                                   (66, 4096, 8), (1000, 512, 2048)])
 def test_fused_matmul_dequantize_swiglu(quest, dtype, shape):
     """The gate/up GEMM with silu(gate) * up in its epilogue = the plain fused GEMM on the same (interleaved) weight
     rows followed by the activation kernel's own SwiGLU, bit for bit; and within 2 ulp of torch's CPU expression on the
