@@ -1085,11 +1085,12 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
 // Between the weight-streaming kernel (a handful of tokens) and the large tiles (thousands) there are too few
 // 256-token tiles to fill the chip, and a large tile that is one or two channel units wide leaves a lone wave per
 // SIMD issuing a few hundred instructions per stage around four multiplications.  Here a workgroup of eight waves
-// owns 64 tokens x 64 channels: waves 0-3 and 4-7 each hold the four 32 x 32 quadrants and split K between them
-// (the first and the second k-pair of every 128-k sub-stage; summed through LDS at the end), which gives every SIMD
-// two waves of a tile and, with two or more tiles per CU, four or more.  Operands travel as in the large-tile
-// kernel: packed bytes HBM -> LDS by direct loads (stages of 256 k = two sub-stages of 64-byte rows, each wave
-// bringing 16 token or channel rows), 16 packed bytes per lane per k-pair, split into the int8 vectors of
+// owns 64 tokens x 64 channels and splits K four ways: wave (q, c) multiplies all 64 tokens by channel half c over
+// k-pair q of every 256-k stage (two accumulators; 9 nibble-splitting operations per MFMA instead of 12 for a
+// 32 x 32 quadrant per wave).  Every SIMD has two waves of a tile and, with two or more tiles per CU, four or more.
+// The four partial sums meet in LDS at the end, and all eight waves share the epilogue.  Operands travel as in the
+// large-tile kernel: packed bytes HBM -> LDS by direct loads (stages of 256 k = two sub-stages of 64-byte rows,
+// each wave bringing 16 token or channel rows), 16 packed bytes per lane per k-pair, split into the int8 vectors of
 // 16 * even-k and 16 * odd-k nibbles for two MFMA k-steps.
 namespace small {
 
@@ -1098,7 +1099,7 @@ constexpr int kRowB = 64;                         // packed bytes per row per su
 constexpr int kHalfB = (kTok + kChn) * kRowB;     // 8 KiB: the token rows of a sub-stage, then its channel rows
 constexpr int kStageB = 2 * kHalfB;               // 16 KiB: 256 k
 constexpr int kStages = 4;
-constexpr int kLdsB = kStages * kStageB;          // 64 KiB: two workgroups per CU
+constexpr int kLdsB = kStages * kStageB;          // 64 KiB: two workgroups per CU; also holds the eight partial tiles
 
 template <int OUT, bool GLU>
 __global__ void __launch_bounds__(512, 4)
@@ -1135,16 +1136,17 @@ gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, 
                                                  kt * 128 + 64, 0, 0);
     };
 
-    // ---- operand reads: row li of the wave's 32 token / channel rows, 16-byte chunk 2 kh + lg of the 64-byte row
-    const int kh = wave >> 2, tr = (wave >> 1) & 1, tc = wave & 1;
+    // ---- operand reads: k-pair kq of the stage = 16-byte chunk 2 (kq & 1) + lg of the 64-byte rows of sub-stage
+    // kq >> 1; row li of each of the two token sub-tiles and of the wave's 32 channel rows
+    const int kq = wave >> 1, tc = wave & 1;
     const int li = lane & 31, lg = lane >> 5;
-    const int rd_x = ((2 * kh + lg) ^ ((li >> 2) & 3)) * 16;
-    const int rd_t = (tr * 32 + li) * kRowB + rd_x;
+    const int rd_x = (kq >> 1) * kHalfB + ((2 * (kq & 1) + lg) ^ ((li >> 2) & 3)) * 16;
+    const int rd_t = li * kRowB + rd_x;
     const int rd_c = (kTok + tc * 32 + li) * kRowB + rd_x;
 
-    v16i acc, acc1;                                      // one per sub-stage: two independent chains of MFMAs
+    v16i acc[2];                                         // token sub-tiles 0 and 1: two independent chains of MFMAs
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = acc1[r] = 0;
+    for (int r = 0; r < 16; r++) acc[0][r] = acc[1][r] = 0;
 
     // Stages 0 .. kStages - 2 in flight before the loop; past the end of K the last stage is fetched again (into a
     // free slot), which keeps the count of outstanding loads uniform.
@@ -1156,58 +1158,58 @@ gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, 
         const int nx = kt + kStages - 1;
         issue(nx < nk ? nx : nk - 1, nx % kStages);
         const uint8_t *sb = lds + (kt % kStages) * kStageB;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const v4i rt = *reinterpret_cast<const v4i *>(sb + h * kHalfB + rd_t);
-            const v4i rc = *reinterpret_cast<const v4i *>(sb + h * kHalfB + rd_c);
-            v4i te, to, ce, co;
-            big::split16(rt, te, to);
-            big::split16(rc, ce, co);
-            if (h == 0) {
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to, acc, 0, 0, 0);
-            } else {
-                acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te, acc1, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to, acc1, 0, 0, 0);
-            }
-        }
+        const v4i r0 = *reinterpret_cast<const v4i *>(sb + rd_t);
+        const v4i r1 = *reinterpret_cast<const v4i *>(sb + rd_t + 32 * kRowB);
+        const v4i rc = *reinterpret_cast<const v4i *>(sb + rd_c);
+        v4i te0, to0, te1, to1, ce, co;
+        big::split16(rc, ce, co);
+        big::split16(r0, te0, to0);
+        big::split16(r1, te1, to1);
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te0, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te1, acc[1], 0, 0, 0);
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to0, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to1, acc[1], 0, 0, 0);
     }
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] += acc1[r];
     big::wait_vmcnt_imm<0>();                            // no direct-to-LDS load may still be writing ...
     big::plain_barrier();                                // ... and nobody still reading when the stages are reused
 
-    // ---- the two K halves: waves 4-7 park their accumulators in LDS, waves 0-3 add them and finish the tile
-    int32_t *red = reinterpret_cast<int32_t *>(lds);     // 4 waves x 16 registers x 64 lanes: 16 KiB
-    if (kh == 1) {
+    // ---- the four K quarters meet in LDS (8 waves x 32 registers x 64 lanes = all 64 KiB); wave (q, c) then finishes
+    // token sub-tile q & 1, channel half c, register groups 2 (q >> 1) and 2 (q >> 1) + 1: 32 tokens x 16 channels
+    int32_t *red = reinterpret_cast<int32_t *>(lds);
 #pragma unroll
-        for (int r = 0; r < 16; r++) red[((wave & 3) * 16 + r) * 64 + lane] = acc[r];
-    }
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[(wave * 32 + b * 16 + r) * 64 + lane] = acc[b][r];
     __syncthreads();
-    if (kh == 1) return;
+    const int tb = kq & 1, pr = kq >> 1;
+    int sum[8];
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] += red[(wave * 16 + r) * 64 + lane];
+    for (int r = 0; r < 8; r++) {
+        sum[r] = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) sum[r] += red[((q * 2 + tc) * 32 + tb * 16 + pr * 8 + r) * 64 + lane];
+    }
 
-    // ---- epilogue: accumulator register r of lane (li, lg) is 256 x the product for token li and channel
-    // 8 (r / 4) + 4 lg + r % 4 of the wave's quadrant
-    const int tok = tok0 + tr * 32 + li;
-    const int cb = ch0 + tc * 32;
+    // ---- epilogue: accumulator register r of lane (li, lg) is 256 x the product for token li of the sub-tile and
+    // channel 8 (r / 4) + 4 lg + r % 4 of the wave's 32; sum[r] is register 8 pr + r
+    const int tok = tok0 + tb * 32 + li;
+    const int cb = ch0 + tc * 32 + pr * 16;              // first channel of the wave's two register groups
     const bool tok_ok = tok < M;
     if constexpr (OUT == OUT_INT32) {
         int32_t *dst = reinterpret_cast<int32_t *>(out) + (size_t)(tok_ok ? tok : 0) * N;
         const bool vec_ok = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;     // 16-byte stores
 #pragma unroll
-        for (int rg = 0; rg < 4; rg++) {
-            const int c = cb + rg * 8 + lg * 4;
+        for (int g = 0; g < 2; g++) {
+            const int c = cb + g * 8 + lg * 4;
             if (!tok_ok) continue;
             if (vec_ok) {
                 if (c < N)
                     *reinterpret_cast<int4 *>(dst + c) =
-                        make_int4(acc[rg * 4] >> 8, acc[rg * 4 + 1] >> 8, acc[rg * 4 + 2] >> 8, acc[rg * 4 + 3] >> 8);
+                        make_int4(sum[g * 4] >> 8, sum[g * 4 + 1] >> 8, sum[g * 4 + 2] >> 8, sum[g * 4 + 3] >> 8);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    if (c + e < N) dst[c + e] = acc[rg * 4 + e] >> 8;
+                    if (c + e < N) dst[c + e] = sum[g * 4 + e] >> 8;
             }
         }
     } else {
@@ -1217,47 +1219,44 @@ gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, 
         // an 8-byte aligned output)
         uint16_t *dst = reinterpret_cast<uint16_t *>(out) + (size_t)(tok_ok ? tok : 0) * (GLU ? N >> 1 : N);
         const bool fast = GLU || ((N & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0);     // 16-byte stores
-        float v[4][4];
+        float v[2][4];
 #pragma unroll
-        for (int rg = 0; rg < 4; rg++) {
+        for (int g = 0; g < 2; g++) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int c = cb + rg * 8 + lg * 4 + e;
+                const int c = cb + g * 8 + lg * 4 + e;
                 const int cc = c < N ? c : N - 1;
                 // the accumulator is 256 C exactly, so 2 C is one arithmetic shift
-                const float lhs = (float)((acc[rg * 4 + e] >> 7) + t_add + b_add[cc]);
+                const float lhs = (float)((sum[g * 4 + e] >> 7) + t_add + b_add[cc]);
                 const float rhs = __fmul_rn(t_half_mul, to_f32<DT>(b_mul[cc]));
-                v[rg][e] = __fmul_rn(lhs, rhs);
+                v[g][e] = __fmul_rn(lhs, rhs);
             }
         }
         if (fast) {
-            // the half-waves trade register groups, so that every lane stores 16 bytes = 8 consecutive channels
-#pragma unroll
-            for (int pr = 0; pr < 2; pr++) {
-                const uint32_t x00 = pack2_rounded_products<DT>(v[2 * pr][0], v[2 * pr][1]);
-                const uint32_t x01 = pack2_rounded_products<DT>(v[2 * pr][2], v[2 * pr][3]);
-                const uint32_t x10 = pack2_rounded_products<DT>(v[2 * pr + 1][0], v[2 * pr + 1][1]);
-                const uint32_t x11 = pack2_rounded_products<DT>(v[2 * pr + 1][2], v[2 * pr + 1][3]);
-                // lower half-wave: group 2 pr complete; upper half-wave: group 2 pr + 1 complete
-                const auto s0 = __builtin_amdgcn_permlane32_swap(x00, x10, false, false);
-                const auto s1 = __builtin_amdgcn_permlane32_swap(x01, x11, false, false);
-                const int c = cb + (2 * pr + lg) * 8;
-                if constexpr (GLU) {
-                    // the lane holds four gate rows, then the four up rows of the same outputs
-                    if (tok_ok && c < N)
-                        *reinterpret_cast<uint2 *>(dst + (c >> 1)) =
-                            make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
-                } else if (tok_ok && c < N) {
-                    *reinterpret_cast<uint4 *>(dst + c) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
-                }
+            // the half-waves trade register groups, so that every lane stores 16 bytes = 8 consecutive channels:
+            // lower half-wave group 0 complete, upper half-wave group 1
+            const uint32_t x00 = pack2_rounded_products<DT>(v[0][0], v[0][1]);
+            const uint32_t x01 = pack2_rounded_products<DT>(v[0][2], v[0][3]);
+            const uint32_t x10 = pack2_rounded_products<DT>(v[1][0], v[1][1]);
+            const uint32_t x11 = pack2_rounded_products<DT>(v[1][2], v[1][3]);
+            const auto s0 = __builtin_amdgcn_permlane32_swap(x00, x10, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(x01, x11, false, false);
+            const int c = cb + lg * 8;
+            if constexpr (GLU) {
+                // the lane holds four gate rows, then the four up rows of the same outputs
+                if (tok_ok && c < N)
+                    *reinterpret_cast<uint2 *>(dst + (c >> 1)) =
+                        make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
+            } else if (tok_ok && c < N) {
+                *reinterpret_cast<uint4 *>(dst + c) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
             }
         } else if (!GLU && tok_ok) {
 #pragma unroll
-            for (int rg = 0; rg < 4; rg++)
+            for (int g = 0; g < 2; g++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const int c = cb + rg * 8 + lg * 4 + e;
-                    if (c < N) dst[c] = (uint16_t)from_f32<DT>(v[rg][e]);
+                    const int c = cb + g * 8 + lg * 4 + e;
+                    if (c < N) dst[c] = (uint16_t)from_f32<DT>(v[g][e]);
                 }
         }
     }
