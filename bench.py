@@ -13,6 +13,7 @@ are converted).  The JSON line also carries
   roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
                      outlier channels) against the HBM peak,
   decode             the layer at M in {1, 8, 16}: the weight-streaming GEMM alone and with the activation kernel,
+  few_hundred_tokens the same at M in {128, 256, 512} (the small-tile GEMM),
   forward            the 12-layer Llama of the reference's end-to-end benchmark, dense vs W4A4 vs no-op linears,
   cpu_baseline       the CPU oracle (PyTorch restatement of the reference's `backend='pytorch'`
                      path) on the reference's CPU-runnable case, timed on this host's cores.
@@ -274,9 +275,10 @@ def bench_quantize(_lib, steps, warmup, dev):
             'sustained_at_8x_rows': sustained}
 
 
-def bench_decode(_lib, dev):
-    """The layer at M in {1, 8, 16}: weights rotate through copies totalling more than the Infinity Cache so that they
-    stream from HBM; bare C-ABI launches, the GEMM alone and the activation kernel + GEMM pair."""
+def bench_decode(_lib, dev, ms=(1, 8, 16)):
+    """The layer at a few token counts M (default: the decode shapes {1, 8, 16}): weights rotate through copies
+    totalling more than the Infinity Cache so that they stream from HBM; bare C-ABI launches, the GEMM alone and the
+    activation kernel + GEMM pair."""
     out = []
     lib = _lib.load()
     dtype = torch.float16
@@ -287,7 +289,7 @@ def bench_decode(_lib, dev):
         ws = [torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.uint8).to(dev) for _ in range(n_w)]
         w_scale = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
         w_add = torch.randint(-500, 500, (n, 1), generator=g, dtype=torch.int32).to(dev)
-        for m in (1, 8, 16):
+        for m in ms:
             x = torch.randn(m, k, generator=g).to(dtype).to(dev)
             a_scale = torch.empty(m, 1, dtype=dtype, device=dev)
             a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
@@ -313,7 +315,8 @@ def bench_decode(_lib, dev):
             wbytes = n * k // 2
             out.append({'M': m, 'K': k, 'N': n, 'gemm_us': round(gemm_us, 2), 'layer_us': round(layer_us, 2),
                         'weight_GBs': round(wbytes / gemm_us / 1e3, 1),
-                        'frac_hbm': round(wbytes / gemm_us / 1e3 / HBM_PEAK_GBS, 4)})
+                        'frac_hbm': round(wbytes / gemm_us / 1e3 / HBM_PEAK_GBS, 4),
+                        'TOPS': round(2.0 * m * n * k / gemm_us / 1e6, 1)})
     return out
 
 
@@ -443,6 +446,7 @@ def main():
     rq = bench_quantize(_lib, max(args.steps, 100), args.warmup, dev)
     lin = bench_linear(quest, _lib, args.steps, args.warmup, dev)
     dec = bench_decode(_lib, dev)
+    few_hundred = bench_decode(_lib, dev, ms=(128, 256, 512))
     fwd = None if args.no_forward else bench_forward(dev)
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
@@ -469,7 +473,7 @@ def main():
         'gemm_tops_on_quantized_activations': 2.0 * 4096 * 4096 * 11008 / (lin['gemm_quantized_acts_ms'] * 1e-3) / 1e12,
         'quantize_us_in_step': lin['quant_ms'] * 1e3,
         'quantize_GBs': rq['achieved'],
-        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'forward': fwd, 'cpu_baseline': cpu,
+        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'few_hundred_tokens': few_hundred, 'forward': fwd, 'cpu_baseline': cpu,
     }
     print(json.dumps(line))
 

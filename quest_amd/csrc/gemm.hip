@@ -1309,8 +1309,12 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 // A few hundred tokens: small tiles, while there are at most four of them per CU (beyond that the large tiles' operand
 // reuse wins), or eight where M would leave the last 256-token tile mostly empty.  Measured against the other kernels
 // over M from 65 to 2048 with (K, N) from (1024, 3072) to (8192, 8192): 1.2 to 2.6 x faster where this picks it.
+// Up to 64 tokens the weight-streaming kernel is the faster one while there are few channels or one token tile; with
+// thousands of channels and more than one (two at N = 8192) of its 16-token tiles, one small tile of 64 tokens per
+// 64 channels is up to 2 x faster (measured at N from 8192 to 28672).
 static bool small_tiles_pay(int M, int K, int N) {
-    if ((K & 255) != 0 || M <= 64) return false;
+    if ((K & 255) != 0) return false;
+    if (M <= 64) return M > 16 && N >= 8192 && (M > 32 || N > 8192);
     const long tiles = (long)((M + small::kTok - 1) / small::kTok) * ((N + small::kChn - 1) / small::kChn);
     const long per_cu = (tiles + device_cu_count() - 1) / device_cu_count();
     return per_cu <= 4 || (per_cu <= 8 && M < 1024 && (M & 255) != 0);

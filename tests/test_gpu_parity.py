@@ -149,6 +149,8 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                # counts that take the element-wise epilogue, one and several tiles per CU, a single 256-k stage
                (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048), (66, 4096, 8),
                (640, 2816, 1024),
+               # ... and a few tens of tokens with thousands of channels
+               (40, 256, 8200), (64, 512, 11008), (17, 256, 11010), (33, 256, 8192),
                # the same token counts with K % 256 != 0 (large tiles one or two channel units wide)
                (200, 384, 512), (300, 640, 1000)]
 
@@ -183,7 +185,7 @@ def test_matmul_int32_extreme_codes(quest):
                                    (4096, 256, 2048), (16384, 128, 2048),
                                    # a few hundred tokens, K % 256 == 0 (small tiles): ragged tiles, vector and element-wise stores
                                    (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048),
-                                   (66, 4096, 8), (640, 2816, 1024),
+                                   (66, 4096, 8), (640, 2816, 1024), (40, 256, 8200), (64, 512, 11008), (17, 256, 11010),
                                    # ... and K % 256 != 0 (narrow large tiles)
                                    (200, 384, 512), (300, 640, 1000)])
 def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
