@@ -13,7 +13,7 @@ are converted).  The JSON line also carries
   roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
                      outlier channels) against the HBM peak,
   decode             the layer at M in {1, 8, 16}: the weight-streaming GEMM alone and with the activation kernel,
-  few_hundred_tokens the same at M in {128, 256, 512} (the small-tile GEMM),
+  few_hundred_tokens the same at M in {128, 256, 384} (the small-tile GEMM),
   forward            the 12-layer Llama of the reference's end-to-end benchmark, dense vs W4A4 vs no-op linears,
   cpu_baseline       the CPU oracle (PyTorch restatement of the reference's `backend='pytorch'`
                      path) on the reference's CPU-runnable case, timed on this host's cores.
@@ -41,8 +41,8 @@ INT8_MFMA_PEAK_TOPS = 5000.0
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
 # scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
-TRAFFIC_GEMM_BYTES = 344227505
-TRAFFIC_QUANTIZE_BYTES = 84239145
+TRAFFIC_GEMM_BYTES = 344287346
+TRAFFIC_QUANTIZE_BYTES = 84237836
 
 
 def event_pairs(n):
@@ -446,7 +446,7 @@ def main():
     rq = bench_quantize(_lib, max(args.steps, 100), args.warmup, dev)
     lin = bench_linear(quest, _lib, args.steps, args.warmup, dev)
     dec = bench_decode(_lib, dev)
-    few_hundred = bench_decode(_lib, dev, ms=(128, 256, 512))
+    few_hundred = bench_decode(_lib, dev, ms=(128, 256, 384))
     fwd = None if args.no_forward else bench_forward(dev)
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
