@@ -151,6 +151,9 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                (640, 2816, 1024),
                # ... and a few tens of tokens with thousands of channels
                (40, 256, 8200), (64, 512, 11008), (17, 256, 11010), (33, 256, 8192),
+               # four 64 x 64 tiles per CU = one round of 128 x 128 tiles (ragged in both directions); one tile per
+               # workgroup of the large-tile kernel, cut along single token tiles
+               (1000, 512, 4090), (1536, 256, 4096), (768, 128, 8200), (1300, 384, 4100),
                # the same token counts with K % 256 != 0 (large tiles one or two channel units wide)
                (200, 384, 512), (300, 640, 1000)]
 
@@ -186,6 +189,7 @@ def test_matmul_int32_extreme_codes(quest):
                                    # a few hundred tokens, K % 256 == 0 (small tiles): ragged tiles, vector and element-wise stores
                                    (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048),
                                    (66, 4096, 8), (640, 2816, 1024), (40, 256, 8200), (64, 512, 11008), (17, 256, 11010),
+                                   (1000, 512, 4090), (1536, 256, 4096), (768, 128, 8200), (1300, 384, 4100),
                                    # ... and K % 256 != 0 (narrow large tiles)
                                    (200, 384, 512), (300, 640, 1000)])
 def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
@@ -209,7 +213,7 @@ def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768, 224), (66, 128, 8), (200, 256, 512), (300, 256, 1000), (16390, 256, 1000),
                                    (16384, 128, 2048), (4096, 128, 4104), (200, 384, 512), (130, 1024, 4104),
-                                   (66, 4096, 8), (1000, 512, 2048)])
+                                   (66, 4096, 8), (1000, 512, 2048), (1000, 512, 4088), (1536, 256, 4096), (768, 128, 8200)])
 def test_fused_matmul_dequantize_swiglu(quest, dtype, shape):
     """The gate/up GEMM with silu(gate) * up in its epilogue = the plain fused GEMM on the same (interleaved) weight
     rows followed by the activation kernel's own SwiGLU, bit for bit; and within 2 ulp of torch's CPU expression on the
