@@ -20,6 +20,7 @@
 // The weight rows feed the MFMA "A" side, so a lane ends up with four consecutive output channels
 // of one token and stores them as one 8- or 16-byte vector.
 #include "common.h"
+#include <type_traits>
 
 namespace quest {
 
@@ -865,26 +866,39 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         // LDS once.  Two per CU: token sub-tile outside, so that the stores of consecutive iterations complete whole
         // 128-byte lines of the same rows (measured -3..-6 % run time at short K; nothing for the wide shape).
         constexpr bool kTokOuter = C::kWgPerCu > 1;
-        int adds[16];
-        float muls[16];
+        // the 16 channel scale values of this lane per unit; in token-outer order all units are unpacked up front (the
+        // main loop's fragment registers are free here) instead of once per token sub-tile
+        constexpr int kSets = kTokOuter ? NAX : 1;
+        int adds_u[kSets][16];
+        float muls_u[kSets][16];
+        auto load_scales = [&](int a, int (&adds)[16], float (&muls)[16]) {
+#pragma unroll
+            for (int rg = 0; rg < 4; rg++) {
+                const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;      // channel inside the tile
+                const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
+                const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
+                adds[rg * 4 + 0] = va.x; adds[rg * 4 + 1] = va.y; adds[rg * 4 + 2] = va.z; adds[rg * 4 + 3] = va.w;
+                muls[rg * 4 + 0] = lo_f32<DT>(vm.x); muls[rg * 4 + 1] = hi_f32<DT>(vm.x);
+                muls[rg * 4 + 2] = lo_f32<DT>(vm.y); muls[rg * 4 + 3] = hi_f32<DT>(vm.y);
+            }
+        };
+        if constexpr (OUT != OUT_INT32 && kTokOuter) {
+#pragma unroll
+            for (int a = 0; a < NA; a++) load_scales(a, adds_u[a], muls_u[a]);
+        }
+        // interior tiles (the common case) store without the per-lane bounds tests and their exec-mask branches
+        auto convert_and_store = [&](auto guarded_tag) {
+        constexpr bool kGuard = decltype(guarded_tag)::value;
 #pragma unroll
         for (int o = 0; o < (kTokOuter ? TB : NA); o++) {
 #pragma unroll
           for (int i = 0; i < (kTokOuter ? NA : TB); i++) {
             const int a = kTokOuter ? i : o, b = kTokOuter ? o : i;
-            if constexpr (OUT != OUT_INT32) {
-              if (kTokOuter || i == 0) {
-#pragma unroll
-                for (int rg = 0; rg < 4; rg++) {
-                    const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;      // channel inside the tile
-                    const int4 va = *reinterpret_cast<const int4 *>(v_add + cl);
-                    const uint2 vm = *reinterpret_cast<const uint2 *>(v_mul + cl);
-                    adds[rg * 4 + 0] = va.x; adds[rg * 4 + 1] = va.y; adds[rg * 4 + 2] = va.z; adds[rg * 4 + 3] = va.w;
-                    muls[rg * 4 + 0] = lo_f32<DT>(vm.x); muls[rg * 4 + 1] = hi_f32<DT>(vm.x);
-                    muls[rg * 4 + 2] = lo_f32<DT>(vm.y); muls[rg * 4 + 3] = hi_f32<DT>(vm.y);
-                }
-              }
+            if constexpr (OUT != OUT_INT32 && !kTokOuter) {
+              if (i == 0) load_scales(a, adds_u[0], muls_u[0]);
             }
+            const int (&adds)[16] = adds_u[kTokOuter ? a : 0];
+            const float (&muls)[16] = muls_u[kTokOuter ? a : 0];
             {
                 const bool tok_ok = tok0 + tok_e + b * 32 + li_e < M;
                 uint8_t *dst = out_lane + ((size_t)b * 32 * n_out + a * kOutPerUnit) * kEs;
@@ -892,7 +906,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
 #pragma unroll
                     for (int rg = 0; rg < 4; rg++) {
                         const int cl = (unit0 + a) * 32 + rg * 8 + lg_e * 4;
-                        if (tok_ok && ch0 + cl < N)
+                        if (!kGuard || (tok_ok && ch0 + cl < N))
                             *reinterpret_cast<int4 *>(dst + (rg * 8 + lg_e * 4) * 4) =
                                 make_int4(acc[a][b][rg * 4] >> 8, acc[a][b][rg * 4 + 1] >> 8, acc[a][b][rg * 4 + 2] >> 8,
                                           acc[a][b][rg * 4 + 3] >> 8);
@@ -922,10 +936,10 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                             // The weight rows come interleaved in eights, four gate rows then the four up rows of the same
                             // outputs: after the swap a lane holds exactly such an eight, gates in (s0[0], s1[0]), ups in
                             // (s0[1], s1[1]), and stores dtype(dtype(silu(gate)) * up) for its four outputs.
-                            if (tok_ok && ch0 + cl < N)
+                            if (!kGuard || (tok_ok && ch0 + cl < N))
                                 *reinterpret_cast<uint2 *>(dst + (2 * pr + lg_e) * 8) =
                                     make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
-                        } else if (tok_ok && ch0 + cl < N) {
+                        } else if (!kGuard || (tok_ok && ch0 + cl < N)) {
                             *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
                         }
                     }
@@ -933,6 +947,8 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             }
           }
         }
+        };
+        if (interior) convert_and_store(std::false_type{}); else convert_and_store(std::true_type{});
     } else if (NA > 0 && !GLU) {
         // generic path (N not a multiple of 8 / 4): element-wise stores straight from the accumulators
 #pragma unroll
