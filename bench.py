@@ -41,8 +41,8 @@ INT8_MFMA_PEAK_TOPS = 5000.0
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
 # scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
-TRAFFIC_GEMM_BYTES = 344287346
-TRAFFIC_QUANTIZE_BYTES = 84237836
+TRAFFIC_GEMM_BYTES = 343050684
+TRAFFIC_QUANTIZE_BYTES = 84238194
 
 
 def event_pairs(n):
