@@ -1466,8 +1466,8 @@ static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int3
     if (small_shape == 64) return gemm_launch_small<small::Tile64, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if (small_shape == 128) return gemm_launch_small<small::Tile128, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     // a handful of tokens: the weight-streaming kernel
-    // (up to 64 of them always; where K rules out the small tiles, up to 128 while its N / 16 workgroups still run
-    // as one round: twice as fast as large tiles that would be half empty)
+    // (up to 64 of them unless the small tiles took the call above; where K rules those out, up to 128 while its
+    // N / 16 workgroups still run as one round: twice as fast as large tiles that would be half empty)
     if (M <= 64 || (M <= 128 && N <= 8192)) {
         const int rc = launch_gemm_decode(OUT, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
         if (rc != QUEST_ERR_UNSUPPORTED) return rc;
