@@ -9,7 +9,14 @@
 // gemm-quest/quest/fused_matmul_dequantize_kernel.cu:4-57 with the functor
 // gemm-quest/include/symmetric/epilogue/thread/linear_combination_dequant.h:122-185).
 //
-// Design.  A workgroup of four waves owns a 256-token x 256-channel tile; each wave a 128 x 128
+// Kernels in this file, chosen by shape in gemm_launch (the weight-streaming kernel for a handful of tokens is in
+// gemm_decode.hip); all give bit-identical results:
+//   gemm_w4a4_staged_kernel   K % 32 == 0: operands staged through registers into int8 LDS tiles (described next);
+//   gemm_w4a4_stream_kernel   K % 128 == 0, odd M or N: packed bytes straight into LDS, plain loop;
+//   gemm_w4a4_big_kernel      K % 128 == 0: the prefill kernel, persistent 256 x 256 or 256 x 128 tiles;
+//   gemm_w4a4_small_kernel    K % 256 == 0, a few hundred tokens: 64 x 64 or 128 x 128 tiles, K split inside the workgroup.
+//
+// The staged kernel.  A workgroup of four waves owns a 256-token x 256-channel tile; each wave a 128 x 128
 // quarter held as 4 x 4 accumulators of v_mfma_i32_32x32x32_i8.  K advances 128 elements per
 // stage.  Packed bytes go HBM -> registers (16 B per lane), are split there into two int8 vectors
 // holding 16 * nibble -- `w & 0xF0F0F0F0` is 16 * (odd-k nibbles), `(w << 4) & 0xF0F0F0F0` is
