@@ -129,7 +129,7 @@ int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uint8_t *x_int
  * dtype-rounded outputs the plain entry point would have written (silu(g) = g / (1 + exp(-g)) in fp32;
  * src/models/llama.py:117-118).  The (size_m, 2 H) tensor is never written.  No counterpart in the reference, which
  * runs two GEMMs and the torch expression.  size_n % 8 == 0; QUEST_ERR_UNSUPPORTED unless size_k % 128 == 0,
- * size_m > 64 and even (the caller then uses the plain entry point and applies the unit itself).
+ * size_m > 64 (the caller then uses the plain entry point and applies the unit itself).
  */
 int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
                                                     const int32_t *vec_a_add, const int32_t *vec_b_add,

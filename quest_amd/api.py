@@ -67,7 +67,7 @@ def fused_matmul_dequantize_swiglu_int4_int4t(
 ) -> torch.Tensor:
     """The gate/up GEMM of a SwiGLU MLP with `silu(gate) * up` (src/models/llama.py:117-118 of the reference) applied
     in its epilogue: mat_b (2 H, K/2) and the vec_b_* hold the rows in `swiglu_interleave_rows` order; returns (M, H).
-    Raises RuntimeError (QUEST_ERR_UNSUPPORTED) for M <= 64, odd M or K % 128 != 0."""
+    Raises RuntimeError (QUEST_ERR_UNSUPPORTED) for M <= 64 or K % 128 != 0."""
     m, n = mat_a.size(0), mat_b.size(0)
     if out is None:
         out = torch.empty(m, n // 2, dtype=vec_a_mul.dtype, device=mat_a.device)

@@ -12,7 +12,7 @@
 // Kernels in this file, chosen by shape in gemm_launch (the weight-streaming kernel for a handful of tokens is in
 // gemm_decode.hip); all give bit-identical results:
 //   gemm_w4a4_staged_kernel   K % 32 == 0: operands staged through registers into int8 LDS tiles (described next);
-//   gemm_w4a4_stream_kernel   K % 128 == 0, odd M or N: packed bytes straight into LDS, plain loop;
+//   gemm_w4a4_stream_kernel   K % 128 == 0, scale vectors not 4-byte aligned: packed bytes straight into LDS, plain loop;
 //   gemm_w4a4_big_kernel      K % 128 == 0: the prefill kernel, persistent 256 x 256 or 256 x 128 tiles;
 //   gemm_w4a4_small_kernel    K % 256 == 0, a few hundred tokens: 64 x 64 or 128 x 128 tiles, K split inside the workgroup.
 //
@@ -1059,9 +1059,12 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     ldr.act = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, M * kbytes, 0x00020000);
     ldr.wgt = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, N * kbytes, 0x00020000);
     ldr.badd = __builtin_amdgcn_make_buffer_rsrc((void *)b_add, 0, N * 4, 0x00020000);
-    ldr.bmul = __builtin_amdgcn_make_buffer_rsrc((void *)b_mul, 0, N * 2, 0x00020000);
+    // the 16-bit scale vectors travel two per dword: an odd count ends with half a dword, which must still count as in
+    // range (the dword lies inside the vector's last aligned word, so nothing outside its memory is touched; the
+    // upper half belongs to a row that does not exist and is never used)
+    ldr.bmul = __builtin_amdgcn_make_buffer_rsrc((void *)b_mul, 0, (N * 2 + 2) & ~3, 0x00020000);
     ldr.aadd = __builtin_amdgcn_make_buffer_rsrc((void *)a_add, 0, M * 4, 0x00020000);
-    ldr.amul = __builtin_amdgcn_make_buffer_rsrc((void *)a_mul, 0, M * 2, 0x00020000);
+    ldr.amul = __builtin_amdgcn_make_buffer_rsrc((void *)a_mul, 0, (M * 2 + 2) & ~3, 0x00020000);
     ldr.kbytes = kbytes;
     ldr.nk = K / 128;
     ldr.wave = wave;
@@ -1479,8 +1482,8 @@ static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int3
         const int rc = launch_gemm_decode(OUT, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
         if (rc != QUEST_ERR_UNSUPPORTED) return rc;
     }
-    // the large-tile kernel fetches the 16-bit scale vectors two per dword: even M, N and 4-byte aligned vectors
-    if ((K & 127) == 0 && M > 64 && (N & 1) == 0 && (M & 1) == 0 && aligned(b_mul, 4) && aligned(a_mul, 4))
+    // the large-tile kernel fetches the 16-bit scale vectors two per dword: 4-byte aligned vectors
+    if ((K & 127) == 0 && M > 64 && aligned(b_mul, 4) && aligned(a_mul, 4))
         return gemm_launch_large<OUT, false>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
@@ -1523,7 +1526,7 @@ extern "C" int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, cons
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (size_n & 7) return QUEST_ERR_BAD_SHAPE;                      // whole eights of weight rows: four gates, four ups
     // only the large-tile kernel has this epilogue
-    if ((size_k & 127) != 0 || size_m <= 64 || (size_m & 1) != 0 || !aligned(vec_b_mul, 4) || !aligned(vec_a_mul, 4) ||
+    if ((size_k & 127) != 0 || size_m <= 64 || !aligned(vec_b_mul, 4) || !aligned(vec_a_mul, 4) ||
         !aligned(mat_d, 8))
         return QUEST_ERR_UNSUPPORTED;
     if (dtype == QUEST_DTYPE_BF16)

@@ -111,7 +111,7 @@ class LlamaMLP(nn.Module):
         """silu(w1 x) * w2 x, (M, hidden), from the codes of x; the gated unit runs in the GEMM's epilogue when that
         kernel takes the shape, otherwise in the torch expression on the plain GEMM's output."""
         m = a_int_packed.size(0)
-        if self.glu is not None and m > 64 and m % 2 == 0 and a_int_packed.size(1) % 64 == 0 and self.w12.bias is None:
+        if self.glu is not None and m > 64 and a_int_packed.size(1) % 64 == 0 and self.w12.bias is None:
             w_packed, w_scale, w_add = self.glu
             return quest.fused_matmul_dequantize_swiglu_int4_int4t(a_int_packed, w_packed, a_int_row_sum, w_add, a_scale, w_scale)
         gate_up = self.w12.forward_quantized(a_scale, a_int_packed, a_int_row_sum)

@@ -154,6 +154,8 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                # four 64 x 64 tiles per CU = one round of 128 x 128 tiles (ragged in both directions); one tile per
                # workgroup of the large-tile kernel, cut along single token tiles
                (1000, 512, 4090), (1536, 256, 4096), (768, 128, 8200), (1300, 384, 4100),
+               # odd token and channel counts in the large-tile kernel (the 16-bit scale vectors end with half a dword)
+               (301, 384, 512), (1001, 128, 96), (4097, 128, 1031), (777, 1152, 4100),
                # the same token counts with K % 256 != 0 (large tiles one or two channel units wide)
                (200, 384, 512), (300, 640, 1000)]
 
@@ -190,6 +192,8 @@ def test_matmul_int32_extreme_codes(quest):
                                    (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048),
                                    (66, 4096, 8), (640, 2816, 1024), (40, 256, 8200), (64, 512, 11008), (17, 256, 11010),
                                    (1000, 512, 4090), (1536, 256, 4096), (768, 128, 8200), (1300, 384, 4100),
+                                   # odd token and channel counts in the large-tile kernel
+                                   (301, 384, 512), (1001, 128, 96), (4097, 128, 1031), (777, 1152, 4100),
                                    # ... and K % 256 != 0 (narrow large tiles)
                                    (200, 384, 512), (300, 640, 1000)])
 def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
@@ -213,7 +217,8 @@ def test_fused_matmul_dequantize_bit_exact(quest, dtype, shape):
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('shape', [(160, 768, 224), (66, 128, 8), (200, 256, 512), (300, 256, 1000), (16390, 256, 1000),
                                    (16384, 128, 2048), (4096, 128, 4104), (200, 384, 512), (130, 1024, 4104),
-                                   (66, 4096, 8), (1000, 512, 2048), (1000, 512, 4088), (1536, 256, 4096), (768, 128, 8200)])
+                                   (66, 4096, 8), (1000, 512, 2048), (1000, 512, 4088), (1536, 256, 4096), (768, 128, 8200),
+                                   (201, 384, 512), (4099, 128, 1032)])
 def test_fused_matmul_dequantize_swiglu(quest, dtype, shape):
     """The gate/up GEMM with silu(gate) * up in its epilogue = the plain fused GEMM on the same (interleaved) weight
     rows followed by the activation kernel's own SwiGLU, bit for bit; and within 2 ulp of torch's CPU expression on the
