@@ -74,12 +74,23 @@ class DenseLinear:
         return F.linear(x, self.weight)
 
 
+class FakeQuantLinear:
+    """The layer a QuEST-trained checkpoint is evaluated with (src/eval_hswag.py:156-217 of the reference): both
+    operands fake-quantised in the rotated space, dense fp32 product, result in the activation dtype."""
+
+    def __init__(self, weight: torch.Tensor, use_hadamard: bool = True):
+        self.weight = weight
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        return qo.fake_quant_linear(x, self.weight).to(x.dtype)
+
+
 def forward(weights: dict, idx: torch.Tensor, n_layer: int, n_head: int, eps: float, use_hadamard: bool = True,
             all_logits: bool = True, linear: str = 'w4a4') -> torch.Tensor:
     """Logits for ids (B, T).  `weights` maps the reference's parameter names (`transformer.wte.weight`,
     `transformer.h.0.attn.c_attn.weight`, ..., `lm_head.weight`) to CPU tensors in the model dtype.
-    linear = 'w4a4' (packed INT4 layers) or 'dense'."""
-    W4A4Linear = {'w4a4': globals()['W4A4Linear'], 'dense': DenseLinear}[linear]     # noqa: N806
+    linear = 'w4a4' (packed INT4 layers), 'fake_quant' (the training-side evaluation layer) or 'dense'."""
+    W4A4Linear = {'w4a4': globals()['W4A4Linear'], 'dense': DenseLinear, 'fake_quant': FakeQuantLinear}[linear]     # noqa: N806
     wte = weights['transformer.wte.weight']
     b, t = idx.shape
     d = wte.size(1)

@@ -11,8 +11,8 @@
 //
 // Kernels in this file, chosen by shape in gemm_launch (the weight-streaming kernel for a handful of tokens is in
 // gemm_decode.hip); all give bit-identical results:
-//   gemm_w4a4_staged_kernel   K % 32 == 0: operands staged through registers into int8 LDS tiles (described next);
-//   gemm_w4a4_stream_kernel   K % 128 == 0, scale vectors not 4-byte aligned: packed bytes straight into LDS, plain loop;
+//   gemm_w4a4_staged_kernel   K % 32 == 0 (and scale vectors that are not 4-byte aligned): operands staged through
+//                             registers into int8 LDS tiles (described next);
 //   gemm_w4a4_big_kernel      K % 128 == 0: the prefill kernel, persistent 256 x 256 or 256 x 128 tiles;
 //   gemm_w4a4_small_kernel    K % 256 == 0, a few hundred tokens: 64 x 64 or 128 x 128 tiles, K split inside the workgroup.
 //
@@ -237,7 +237,8 @@ gemm_w4a4_staged_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
 static int gemm_check(const void *out, const uint8_t *a, const uint8_t *b, int M, int K, int N) {
     if (!out || !a || !b) return QUEST_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (K & 31)) return QUEST_ERR_BAD_SHAPE;
-    if (K > 131072) return QUEST_ERR_UNSUPPORTED;       // keeps 256 * |C| below 2^31
+    // the accumulators hold 256 C and |C| <= 64 K: K = 131072 with all codes -8 would reach 2^31 exactly
+    if (K >= 131072) return QUEST_ERR_UNSUPPORTED;
     if ((size_t)M * (K / 2) >= (1ull << 31) || (size_t)N * (K / 2) >= (1ull << 31)) return QUEST_ERR_UNSUPPORTED;  // 32-bit row offsets
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(out, 16)) return QUEST_ERR_ALIGNMENT;
     return QUEST_OK;
@@ -254,243 +255,13 @@ static int gemm_launch_staged(void *out, const uint8_t *a, const uint8_t *b, con
 }
 
 
-// =================================================================================================
-// Persistent kernel (K % 128 == 0): packed bytes stay packed in LDS
-// =================================================================================================
-// Two workgroups live on every CU (72 KiB of LDS and 256 registers per lane each), so one's
-// barriers, prologue and epilogue stores overlap the other's matrix work.  A workgroup owns
-// 256 tokens x up to 128 channels; its four waves are stacked along the tokens (64 each) and all
-// read the same channel rows, so any width of 1..4 units of 32 channels costs exactly its share.
-// The grid is persistent: the (token tile, channel unit) space of each XCD's slice of the channels
-// is cut into equal contiguous runs, one per workgroup, which removes the tail a fixed tile grid
-// leaves (11008 channels: 97.7 % balance instead of 89.6 %).
-//
-// Packed bytes go HBM -> LDS directly (global_load_lds_dwordx4, no registers, no ds_write), three
-// stages deep.  A lane reads 16 packed bytes (32 codes) of one row and splits them into the int8
-// vector of 16 * (even-k nibbles) and the one of 16 * (odd-k nibbles): two MFMA k-steps per read.
-namespace stream {
-
-constexpr int kTok = 256;                 // token rows per workgroup tile
-constexpr int kMaxUnits = 4;              // channel units (32 rows each) per workgroup tile
-constexpr int kChn = 32 * kMaxUnits;
-constexpr int kRowB = 64;                 // packed bytes per row per stage = 128 k
-constexpr int kStages = 3;
-constexpr int kStageB = (kTok + kChn) * kRowB;      // 24 KiB
-constexpr int kLdsB = kStages * kStageB;            // 72 KiB
-
-__device__ __forceinline__ void wait_vmcnt(int n) {
-    // gfx9 s_waitcnt immediate: vmcnt in bits [3:0] and [15:14]; expcnt / lgkmcnt left at "no wait"
-    switch (n) {
-        case 0: __builtin_amdgcn_s_waitcnt((0 & 15) | ((0 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-        case 6: __builtin_amdgcn_s_waitcnt((6 & 15) | ((6 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-        case 12: __builtin_amdgcn_s_waitcnt((12 & 15) | ((12 >> 4) << 14) | (7 << 4) | (15 << 8)); break;
-        default: __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8)); break;
-    }
-}
-
+// How a persistent grid divides the (token tile, channel unit) cells among its workgroups.
 struct Schedule {
     int tiles_t;        // token tiles of 256
     int units;          // channel units of 32
     int groups;         // channel super-groups (one per XCD when the grid allows)
-    int row_tiles;      // large-tile kernel: > 0 = one tile per workgroup, this many per token tile of a group (0: runs of cells)
+    int row_tiles;      // > 0: one tile per workgroup, this many per token tile of a group (0: contiguous runs of cells)
 };
-
-__device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        even[d] = (int)(((uint32_t)p[d] << 4) & 0xF0F0F0F0u);
-        odd[d] = (int)((uint32_t)p[d] & 0xF0F0F0F0u);
-    }
-}
-
-// One tile of 256 tokens x 32 W channels: K loop and epilogue, everything unrolled for W.
-template <int OUT, int W>
-__device__ __forceinline__ void stream_tile(uint8_t *lds, void *__restrict__ out, const uint8_t *__restrict__ act,
-                                            const uint8_t *__restrict__ wgt, const int32_t *__restrict__ a_add,
-                                            const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
-                                            const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0) {
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wv = tid >> 6;                // token quarter of the tile
-    const int li = lane & 31;
-    const int lg = lane >> 5;
-    const int kbytes = K >> 1;
-    const int nk = K / 128;
-    // loads: wave wv brings token rows [64 wv, +64) (4 instructions of 16 rows) and channel rows
-    // [32 wv, +32) (2 instructions, skipped when the tile is narrower); lane p of an instruction
-    // takes row p/4, 16-byte chunk p%4, and the 64 lanes fill 1 KiB of LDS in lane order.
-    // The 16-byte chunk c of row r sits at position c ^ ((r >> 2) & 3) of its 64-byte LDS row, so that
-    // 16 consecutive rows read at the same chunk touch 16 different bank groups.
-    const int lrow = lane >> 2;
-    const int lchunk = ((lane & 3) ^ ((lane >> 4) & 3)) * 16;
-    // operand reads: row li of a 32-row sub-tile, bytes [32 j + 16 lg, +16) of the 64-byte stage row
-    int rd_lane[2];
-#pragma unroll
-    for (int j = 0; j < 2; j++) rd_lane[j] = li * kRowB + (((2 * j + lg) ^ ((li >> 2) & 3)) * 16);
-    constexpr int kLoads = 4 + 2;            // per wave per stage (channel loads are issued even if unused)
-
-    uint32_t t_off[4], c_off[2];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        int t = tok0 + wv * 64 + j * 16 + lrow;
-        t = t < M ? t : M - 1;
-        t_off[j] = (uint32_t)t * (uint32_t)kbytes + lchunk;
-    }
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        int c = ch0 + wv * 32 + j * 16 + lrow;
-        c = c < N ? c : N - 1;
-        c_off[j] = (uint32_t)c * (uint32_t)kbytes + lchunk;
-    }
-
-    auto issue_loads = [&](int kt) {
-        const int k_idx = kt < nk ? kt : nk - 1;        // past the end: a harmless re-load keeps the counts uniform
-        const int kb = k_idx * kRowB;
-        uint8_t *sb = lds + (kt % kStages) * kStageB;
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void *)(act + t_off[j] + kb),
-                (__attribute__((address_space(3))) void *)(sb + (wv * 64 + j * 16) * kRowB), 16, 0, 0);
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void *)(wgt + c_off[j] + kb),
-                (__attribute__((address_space(3))) void *)(sb + (kTok + wv * 32 + j * 16) * kRowB), 16, 0, 0);
-    };
-
-    v16i acc[W][2];
-#pragma unroll
-    for (int a = 0; a < W; a++)
-#pragma unroll
-        for (int b = 0; b < 2; b++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
-
-    __builtin_amdgcn_s_barrier();            // every wave is done reading the previous tile's stages
-#pragma unroll
-    for (int s = 0; s < kStages - 1; s++) issue_loads(s);
-
-    for (int kt = 0; kt < nk; kt++) {
-        wait_vmcnt(kLoads * (kStages - 2));  // this wave's share of stage kt has landed
-        __builtin_amdgcn_s_barrier();        // ... and everyone else's; slot (kt-1) % kStages is free again
-        issue_loads(kt + kStages - 1);
-        const uint8_t *sb = lds + (kt % kStages) * kStageB;
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            v4i te[2], to[2];
-#pragma unroll
-            for (int b = 0; b < 2; b++) {
-                const v4i p = *reinterpret_cast<const v4i *>(sb + (wv * 64 + b * 32) * kRowB + rd_lane[j]);
-                split16(p, te[b], to[b]);
-            }
-#pragma unroll
-            for (int a = 0; a < W; a++) {
-                const v4i p = *reinterpret_cast<const v4i *>(sb + (kTok + a * 32) * kRowB + rd_lane[j]);
-                v4i ce, co;
-                split16(p, ce, co);
-#pragma unroll
-                for (int b = 0; b < 2; b++) {
-                    acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ce, te[b], acc[a][b], 0, 0, 0);
-                    acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(co, to[b], acc[a][b], 0, 0, 0);
-                }
-            }
-        }
-    }
-
-    // ---- epilogue: register r of lane (li, lg) is channel 8 (r/4) + 4 lg + r%4, token li -------------
-    const bool vec_ok = (N & 3) == 0;
-#pragma unroll
-    for (int b = 0; b < 2; b++) {
-        const int tok = tok0 + wv * 64 + b * 32 + li;
-        if (tok >= M) continue;
-        int t_add = 0;
-        float t_half_mul = 0.f;
-        if constexpr (OUT != OUT_INT32) {
-            t_add = a_add[tok];
-            t_half_mul = __fmul_rn(0.5f, to_f32<OUT>(a_mul[tok]));
-        }
-#pragma unroll
-        for (int a = 0; a < W; a++) {
-#pragma unroll
-            for (int rg = 0; rg < 4; rg++) {
-                const int ch = ch0 + a * 32 + rg * 8 + lg * 4;
-                if (ch >= N) continue;
-                int c[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) c[e] = acc[a][b][rg * 4 + e] >> 8;
-                const size_t o = (size_t)tok * N + ch;
-                if constexpr (OUT == OUT_INT32) {
-                    int32_t *dst = reinterpret_cast<int32_t *>(out) + o;
-                    if (vec_ok) {
-                        *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (ch + e < N) dst[e] = c[e];
-                    }
-                } else {
-                    uint32_t h[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int che = (ch + e < N) ? ch + e : N - 1;
-                        const float lhs = (float)(c[e] * 2 + t_add + b_add[che]);
-                        const float rhs = __fmul_rn(t_half_mul, to_f32<OUT>(b_mul[che]));
-                        h[e] = from_f32<OUT>(__fmul_rn(lhs, rhs));
-                    }
-                    uint16_t *dst = reinterpret_cast<uint16_t *>(out) + o;
-                    if (vec_ok) {
-                        *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (ch + e < N) dst[e] = (uint16_t)h[e];
-                    }
-                }
-            }
-        }
-    }
-}
-
-template <int OUT>
-__global__ void __launch_bounds__(256, 2)
-gemm_w4a4_stream_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
-                        const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
-                        const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
-                        int M, int N, int K, Schedule sch) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsB];
-
-    // ---- this workgroup's run of (token tile, channel unit) cells ---------------------------------
-    const int grp = blockIdx.x % sch.groups;                 // = XCD when groups == 8
-    const int rank = blockIdx.x / sch.groups;
-    const int per_grp = gridDim.x / sch.groups;
-    const int ug0 = (int)(((long)grp * sch.units) / sch.groups);
-    const int ug1 = (int)(((long)(grp + 1) * sch.units) / sch.groups);
-    const int nug = ug1 - ug0;
-    const long cells = (long)sch.tiles_t * nug;
-    long pos = (cells * rank) / per_grp;
-    const long pos_end = (cells * (rank + 1)) / per_grp;
-
-    while (pos < pos_end) {
-        const int tt = (int)(pos / nug);
-        const int u_in = (int)(pos % nug);
-        long seg_end = (long)(tt + 1) * nug;
-        if (seg_end > pos_end) seg_end = pos_end;
-        int width = (int)(seg_end - pos);
-        if (width > kMaxUnits) width = kMaxUnits;
-        pos += width;
-        const int tok0 = tt * kTok;
-        const int ch0 = (ug0 + u_in) * 32;
-        switch (width) {
-            case 4: stream_tile<OUT, 4>(lds, out, act, wgt, a_add, b_add, a_mul, b_mul, M, N, K, tok0, ch0); break;
-            case 3: stream_tile<OUT, 3>(lds, out, act, wgt, a_add, b_add, a_mul, b_mul, M, N, K, tok0, ch0); break;
-            case 2: stream_tile<OUT, 2>(lds, out, act, wgt, a_add, b_add, a_mul, b_mul, M, N, K, tok0, ch0); break;
-            default: stream_tile<OUT, 1>(lds, out, act, wgt, a_add, b_add, a_mul, b_mul, M, N, K, tok0, ch0); break;
-        }
-    }
-}
-
-}  // namespace stream
 
 
 // =================================================================================================
@@ -1009,7 +780,7 @@ __global__ void __launch_bounds__(256, C::kWgPerCu)
 gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                      const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
                      const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
-                     int M, int N, int K, stream::Schedule sch) {
+                     int M, int N, int K, Schedule sch) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[C::kLdsB];
     // wave-uniform by construction; readfirstlane tells the compiler so, which keeps everything that is
     // updated under `switch (na)` below (cursors, slot numbers, LDS bases) in scalar registers; the empty
@@ -1357,42 +1128,23 @@ gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, 
 
 }  // namespace small
 
-static int device_cu_count() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
+// Compute units of the device the stream belongs to.  Asked for at every launch (two host-side queries, no stream
+// operation, nothing cached): the library keeps no state and a process may drive several devices.
+static int device_cu_count(hipStream_t st) {
+    int dev = 0, cus = 0;
+    if (hipStreamGetDevice(st, &dev) != hipSuccess && hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
     return cus;
-}
-
-template <int OUT>
-static int gemm_launch_stream(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                              const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    stream::Schedule sch;
-    sch.tiles_t = (M + stream::kTok - 1) / stream::kTok;
-    sch.units = (N + 31) / 32;
-    const long cells = (long)sch.tiles_t * sch.units;
-    long grid = 2L * device_cu_count();                     // two co-resident workgroups per CU
-    if (grid > cells) grid = cells;
-    sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
-    sch.row_tiles = 0;
-    stream::gemm_w4a4_stream_kernel<OUT><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
-        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
-    return launch_status();
 }
 
 template <typename C, int OUT, bool GLU = false>
 static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                            const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    stream::Schedule sch;
+    Schedule sch;
     sch.tiles_t = (M + big::kRows - 1) / big::kRows;
     sch.units = (N + 31) / 32;
     const long cells = (long)sch.tiles_t * sch.units;
-    long grid = (long)C::kWgPerCu * device_cu_count();      // persistent: one or two workgroups per CU
+    long grid = (long)C::kWgPerCu * device_cu_count(st);      // persistent: one or two workgroups per CU
     if (grid > cells) grid = cells;
     sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
     sch.row_tiles = 0;
@@ -1425,10 +1177,9 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 // Up to 64 tokens the weight-streaming kernel is the faster one while there are few channels or one token tile; with
 // thousands of channels and more than one (two at N = 8192) of its 16-token tiles, one small tile of 64 tokens per
 // 64 channels is up to 2 x faster (measured at N from 8192 to 28672).
-static int small_tile_shape(int M, int K, int N) {
+static int small_tile_shape(int M, int K, int N, int cus) {
     if ((K & 255) != 0) return 0;
     if (M <= 64) return (M > 16 && N >= 8192 && (M > 32 || N > 8192)) ? 64 : 0;
-    const int cus = device_cu_count();
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
     const long per_cu = (tiles + cus - 1) / cus;
     if (per_cu <= 3) return 64;
@@ -1456,7 +1207,7 @@ static int gemm_launch_small(void *out, const uint8_t *a, const uint8_t *b, cons
 template <int OUT, bool GLU>
 static int gemm_launch_large(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                              const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    const int small_shape = small_tile_shape(M, K, N);
+    const int small_shape = small_tile_shape(M, K, N, device_cu_count(st));
     if (small_shape == 64) return gemm_launch_small<small::Tile64, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if (small_shape == 128) return gemm_launch_small<small::Tile128, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     const int units = (N + 31) / 32;
@@ -1472,7 +1223,7 @@ static int gemm_launch_large(void *out, const uint8_t *a, const uint8_t *b, cons
 template <int OUT>
 static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    const int small_shape = small_tile_shape(M, K, N);
+    const int small_shape = small_tile_shape(M, K, N, device_cu_count(st));
     if (small_shape == 64) return gemm_launch_small<small::Tile64, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     if (small_shape == 128) return gemm_launch_small<small::Tile128, OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     // a handful of tokens: the weight-streaming kernel
@@ -1485,7 +1236,8 @@ static int gemm_launch(void *out, const uint8_t *a, const uint8_t *b, const int3
     // the large-tile kernel fetches the 16-bit scale vectors two per dword: 4-byte aligned vectors
     if ((K & 127) == 0 && M > 64 && aligned(b_mul, 4) && aligned(a_mul, 4))
         return gemm_launch_large<OUT, false>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    if ((K & 127) == 0) return gemm_launch_stream<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    // K % 128 != 0, or scale vectors at odd element offsets (a sliced tensor): the register-staged kernel reads them
+    // element by element
     return gemm_launch_staged<OUT>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
 

@@ -293,8 +293,13 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
     }
     if (packed != nullptr && live) {
         uint32_t *dst = packed + (size_t)row * (K >> 3) + blk * 16 + h * 8;
-        *reinterpret_cast<uint4 *>(dst) = make_uint4(dw[0], dw[1], dw[2], dw[3]);
-        *reinterpret_cast<uint4 *>(dst + 4) = make_uint4(dw[4], dw[5], dw[6], dw[7]);
+        if ((reinterpret_cast<uintptr_t>(packed) & 15) == 0) {           // uniform; rows are whole multiples of 64 bytes
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(dw[0], dw[1], dw[2], dw[3]);
+            *reinterpret_cast<uint4 *>(dst + 4) = make_uint4(dw[4], dw[5], dw[6], dw[7]);
+        } else {                                                          // a view that starts 4 bytes into an allocation
+#pragma unroll
+            for (int t = 0; t < 8; t++) dst[t] = dw[t];
+        }
     }
     if (row_sum != nullptr) {
         if (!live) isum = 0;                    // a dead lane's zeros need not quantise to code 0
@@ -391,8 +396,10 @@ static void launch_dtype(int pre, const Args &a) {
 
 // Launches the matrix-core kernel when it applies (K a multiple of 128 up to 32768 -- 4096 with a producer --, a
 // Hadamard entry the dtype represents exactly); returns QUEST_ERR_UNSUPPORTED otherwise so that the caller can take
-// another path.  pre: 0 none, 1 RMSNorm (norm_w, eps; with add_in the norm of x + add_in, the sum written to
-// sum_out), 2 SiLU(gate) * up with x a (M, 2 K) tensor.
+// another path.  Whether it applies depends on K, the factor and the dtype only -- never on the number of rows or on
+// where the buffers lie -- so that one shape always runs the same arithmetic.
+// pre: 0 none, 1 RMSNorm (norm_w, eps; with add_in the norm of x + add_in, the sum written to sum_out), 2 SiLU(gate) * up
+// with x a (M, 2 K) tensor.
 int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
                                   int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
                                   hipStream_t st, const void *add_in, void *sum_out) {
@@ -400,13 +407,23 @@ int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, fl
     if (K > 32768 || (K & 127) || had_scale <= 0.f || !representable16(had_scale, dtype, &bits)) return QUEST_ERR_UNSUPPORTED;
     if (pre != hq::kPreNone && K > 4096) return QUEST_ERR_UNSUPPORTED;
     const int ldx = pre == hq::kPreSiluMul ? 2 * K : K;
-    if ((long)M * ldx * 2 >= (1L << 31)) return QUEST_ERR_UNSUPPORTED;        // 32-bit buffer offsets
-    if (!aligned(packed, 16) || !aligned(x_had, 8) || !aligned(pre_out, 16) || !aligned(norm_w, 16)) return QUEST_ERR_UNSUPPORTED;
+    if (!aligned(pre_out, 16) || !aligned(norm_w, 16)) return QUEST_ERR_UNSUPPORTED;
     if (add_in != nullptr && (pre != hq::kPreRmsNorm || sum_out == nullptr || !aligned(add_in, 16) || !aligned(sum_out, 16)))
         return QUEST_ERR_UNSUPPORTED;
-    const Args a = {x, norm_w, scale, packed, row_sum, x_had, pre_out, add_in, sum_out, K, M, ldx, bits, eps, st};
-    if (dtype == QUEST_DTYPE_BF16) launch_dtype<0>(pre, a);
-    else launch_dtype<1>(pre, a);
+    // The kernel addresses its input with 32-bit byte offsets: tensors of 2 GiB and more go as several launches of
+    // whole rows (same kernel, same arithmetic, so the result does not depend on where the cut falls).
+    const long max_rows = ((1L << 31) - 1) / ((long)ldx * 2);
+    const size_t es = 2;
+    for (long r0 = 0; r0 < M; r0 += max_rows) {
+        const int rows = (int)(M - r0 < max_rows ? M - r0 : max_rows);
+        auto at = [&](const void *p, size_t row_elems, size_t elem) -> void * {
+            return p == nullptr ? nullptr : (void *)((const uint8_t *)p + (size_t)r0 * row_elems * elem);
+        };
+        const Args a = {at(x, ldx, es), norm_w, at(scale, 1, es), (uint8_t *)at(packed, K / 2, 1), (int32_t *)at(row_sum, 1, 4),
+                        at(x_had, K, es), at(pre_out, K, es), at(add_in, K, es), at(sum_out, K, es), K, rows, ldx, bits, eps, st};
+        if (dtype == QUEST_DTYPE_BF16) launch_dtype<0>(pre, a);
+        else launch_dtype<1>(pre, a);
+    }
     return launch_status();
 }
 

@@ -390,7 +390,8 @@ extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t 
                                             void *stream) {
     if (!x || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
-    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    // the transform works on blocks of 128; without it (had_scale == 0) a row only has to be whole 16-byte chunks
+    if (group_size <= 0 || batch_size <= 0 || (group_size & (had_scale != 0.f ? 127 : 7))) return QUEST_ERR_BAD_SHAPE;
     if (!aligned(x, 16) || !aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
     hipStream_t st = (hipStream_t)stream;
     // rows of up to 32768 with a Hadamard entry the dtype holds exactly: matrix cores; anything else: butterflies
@@ -413,7 +414,8 @@ extern "C" int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uin
     if (scale_rule != QUEST_SCALE_ABSMAX) return QUEST_ERR_BAD_SHAPE;
     if (!x || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
-    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    // the transform works on blocks of 128; without it (had_scale == 0) a row only has to be whole 16-byte chunks
+    if (group_size <= 0 || batch_size <= 0 || (group_size & (had_scale != 0.f ? 127 : 7))) return QUEST_ERR_BAD_SHAPE;
     if (!aligned(x, 16) || !aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == QUEST_DTYPE_BF16)

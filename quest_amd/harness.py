@@ -8,8 +8,6 @@ the HIP kernels; 'pytorch' (the reference's eager-torch twin) is not part of thi
 """
 from __future__ import annotations
 
-import time
-
 import torch
 from torch import nn
 
@@ -126,38 +124,47 @@ def linear_forward(activation, w_int_packed, w_scale, w_add, w_meta_e=None, out=
 
 
 class Linear4bit(nn.Module):
-    """bench_e2e.py:41-70: a linear layer holding packed INT4 weights, built from a randomly
-    initialised nn.Linear of the same shape (the benchmarks never load trained weights)."""
+    """bench_e2e.py:41-70: a linear layer that holds its weight as packed INT4 codes.
+
+    Buffers, as in the reference: `w_int_packed` (N, K/2) uint8, `w_scale` (N, 1), `w_add` (N, 1) int32 and the
+    unused `w_meta_e`; `weight` is a shape-only meta tensor; `bias` is a parameter or None.  The plain constructor
+    packs the weight of a freshly initialised `nn.Linear` (the benchmarks never load trained weights),
+    `from_weight` packs a given one and `empty` leaves the buffers to `load_state_dict`."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None,
                  use_sparse: bool = False, use_hadamard: bool = False, use_noop: bool = False):
         super().__init__()
+        if use_sparse:
+            raise NotImplementedError('4:8-sparse weights are not part of this build')
+        dense = nn.Linear(in_features, out_features, bias=bias, device=device, dtype=dtype)
+        self._configure(use_hadamard, use_noop)
+        self._install(dense.weight.data, dense.bias)
+
+    def _configure(self, use_hadamard: bool, use_noop: bool) -> None:
         self.use_hadamard = use_hadamard
         self.use_noop = use_noop
-        nn_linear = nn.Linear(in_features, out_features, bias=bias, device=device, dtype=dtype)
-        self.bias = nn_linear.bias
-        weight = nn_linear.weight.data
-        self.weight = torch.empty_like(weight, device=torch.device('meta'))
-        w_int_packed, w_scale, w_add, w_meta_e = preprocess_weight(weight=weight, use_sparse=use_sparse,
-                                                                   use_hadamard=use_hadamard)
-        self.register_buffer('w_int_packed', w_int_packed)
-        self.register_buffer('w_scale', w_scale)
-        self.register_buffer('w_add', w_add)
-        self.register_buffer('w_meta_e', w_meta_e)
+
+    def _install(self, weight: torch.Tensor, bias) -> None:
+        """Pack `weight` (N, K) and keep `bias` (a tensor, a parameter or None) as a frozen parameter."""
+        packed, scale, add, _ = preprocess_weight(weight=weight, use_hadamard=self.use_hadamard)
+        self._set_buffers(weight.shape, weight.dtype, packed, scale, add)
+        if bias is None:
+            self.bias = None
+        else:
+            self.bias = nn.Parameter(bias.detach().to(weight.dtype), requires_grad=False)
+
+    def _set_buffers(self, shape, dtype, packed, scale, add) -> None:
+        self.weight = torch.empty(shape, dtype=dtype, device='meta')
+        for name, t in (('w_int_packed', packed), ('w_scale', scale), ('w_add', add), ('w_meta_e', None)):
+            self.register_buffer(name, t)
 
     @classmethod
     def from_weight(cls, weight: torch.Tensor, bias: torch.Tensor = None, use_hadamard: bool = False) -> 'Linear4bit':
         """Pack an existing (N, K) weight instead of a random one."""
         self = cls.__new__(cls)
         nn.Module.__init__(self)
-        self.use_hadamard, self.use_noop = use_hadamard, False
-        self.bias = bias
-        self.weight = torch.empty_like(weight, device=torch.device('meta'))
-        w_int_packed, w_scale, w_add, _ = preprocess_weight(weight=weight, use_hadamard=use_hadamard)
-        self.register_buffer('w_int_packed', w_int_packed)
-        self.register_buffer('w_scale', w_scale)
-        self.register_buffer('w_add', w_add)
-        self.register_buffer('w_meta_e', None)
+        self._configure(use_hadamard, False)
+        self._install(weight, bias)
         return self
 
     @classmethod
@@ -166,13 +173,12 @@ class Linear4bit(nn.Module):
         """A layer of the given shape with unset buffers, to be filled by `load_state_dict` from a packed checkpoint."""
         self = cls.__new__(cls)
         nn.Module.__init__(self)
-        self.use_hadamard, self.use_noop = use_hadamard, False
-        self.bias = nn.Parameter(torch.zeros(out_features, dtype=dtype, device=device)) if bias else None
-        self.weight = torch.empty(out_features, in_features, dtype=dtype, device=torch.device('meta'))
-        self.register_buffer('w_int_packed', torch.zeros(out_features, in_features // 2, dtype=torch.uint8, device=device))
-        self.register_buffer('w_scale', torch.zeros(out_features, 1, dtype=dtype, device=device))
-        self.register_buffer('w_add', torch.zeros(out_features, 1, dtype=torch.int32, device=device))
-        self.register_buffer('w_meta_e', None)
+        self._configure(use_hadamard, False)
+        self._set_buffers((out_features, in_features), dtype,
+                          torch.zeros(out_features, in_features // 2, dtype=torch.uint8, device=device),
+                          torch.zeros(out_features, 1, dtype=dtype, device=device),
+                          torch.zeros(out_features, 1, dtype=torch.int32, device=device))
+        self.bias = nn.Parameter(torch.zeros(out_features, dtype=dtype, device=device), requires_grad=False) if bias else None
         return self
 
     def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None) -> torch.Tensor:
@@ -186,54 +192,66 @@ class Linear4bit(nn.Module):
         return y
 
     def forward(self, x) -> torch.Tensor:
-        if not self.use_noop:
-            a = x.contiguous().flatten(end_dim=-2)
-            y = linear_forward(activation=a, w_int_packed=self.w_int_packed, w_scale=self.w_scale, w_add=self.w_add,
-                               w_meta_e=self.w_meta_e, out=None, use_hadamard=self.use_hadamard)
-            y = y.unflatten(dim=0, sizes=x.shape[:-1])
+        lead, n = x.shape[:-1], self.weight.size(0)
+        rows = x.contiguous().view(-1, x.size(-1))
+        if self.use_noop:
+            # the reference's no-op layer (bench_e2e.py:62-66) still rotates the activations, so that
+            # "int4 minus noop" prices the quantiser and the GEMM only; the rotated tensor is dropped
+            if self.use_hadamard:
+                quest.hadamard128(rows)
+            y = torch.zeros(rows.size(0), n, dtype=x.dtype, device=x.device)
         else:
-            y = torch.zeros(*x.shape[:-1], self.weight.size(0), dtype=x.dtype, device=x.device)
+            y = linear_forward(rows, self.w_int_packed, self.w_scale, self.w_add, self.w_meta_e,
+                               use_hadamard=self.use_hadamard)
         if self.bias is not None:
             y += self.bias
-        return y
+        return y.view(*lead, n)
+
+
+def _elapsed_s(fn, n_iter: int) -> float:
+    """Seconds per call of `fn`, from a pair of HIP events on the current stream around n_iter calls."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(n_iter):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / n_iter
 
 
 @torch.inference_mode()
 def do_bench(f, n_iter: int = 100, n_warmup: int = 10) -> float:
-    """utils.py:789-799: seconds per call, wall clock around a device synchronisation."""
+    """utils.py:789-799: seconds per call of `f` after `n_warmup` untimed calls.  The reference brackets the timed
+    calls with device synchronisations and the host clock; here the bracket is a pair of HIP events on the stream
+    the calls go to, which leaves the host's launch jitter before the first call out of the figure."""
     for _ in range(n_warmup):
         f()
     torch.cuda.synchronize()
-    ts = time.time()
-    for _ in range(n_iter):
-        f()
-    torch.cuda.synchronize()
-    te = time.time()
-    return (te - ts) / n_iter
+    return _elapsed_s(f, n_iter)
 
 
 @torch.inference_mode()
 def do_bench_network(f, M: int, K: int, N: int, dtype: torch.dtype, device: torch.device, n_layers: int = 20,
                      n_warmup: int = 3) -> float:
-    """utils.py:802-835: n_layers back-to-back calls on one aliased workspace, timed eagerly and as a
-    replayed HIP graph; the smaller per-layer time is returned."""
-    workspace = torch.empty(M * max(K, N), dtype=dtype, device=device)
-    activation_in = workspace[:M * K].reshape(M, K)
-    activation_out = workspace[:M * N].reshape(M, N)
+    """utils.py:802-835: `f(activation_in (M, K), activation_out (M, N))` called `n_layers` times back to back on
+    two views of one buffer (so that no call finds a fresh output allocation), timed as plain launches and as one
+    replayed HIP graph; returns the smaller of the two, in seconds per layer."""
+    pool = torch.empty(M * max(K, N), dtype=dtype, device=device)
+    a_in, a_out = pool[:M * K].view(M, K), pool[:M * N].view(M, N)
 
-    def network():
+    def stack():
         for _ in range(n_layers):
-            f(activation_in, activation_out)
+            f(a_in, a_out)
 
-    tf = do_bench(network, n_iter=1, n_warmup=n_warmup)
+    eager_s = do_bench(stack, n_iter=1, n_warmup=n_warmup)
+    capture = torch.cuda.Stream(device=device)
+    capture.wait_stream(torch.cuda.current_stream(device))
     graph = torch.cuda.CUDAGraph()
-    s = torch.cuda.Stream()
-    s.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(s):
+    with torch.cuda.stream(capture):
         for _ in range(n_warmup):
-            network()
-    torch.cuda.current_stream().wait_stream(s)
-    with torch.cuda.graph(graph):
-        network()
-    tg = do_bench(graph.replay, n_iter=1, n_warmup=n_warmup)
-    return min(tf, tg) / n_layers
+            stack()
+        with torch.cuda.graph(graph, stream=capture):
+            stack()
+    torch.cuda.current_stream(device).wait_stream(capture)
+    graph_s = do_bench(graph.replay, n_iter=1, n_warmup=n_warmup)
+    return min(eager_s, graph_s) / n_layers

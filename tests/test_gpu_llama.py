@@ -136,3 +136,57 @@ def test_packed_checkpoint_serves_the_same_logits(llama, tmp_path):
     ids = torch.randint(0, cfg.vocab_size, (2, 48), generator=torch.Generator().manual_seed(6)).to(DEV)
     with torch.no_grad():
         assert torch.equal(model(ids, all_logits=True)['logits'], back(ids, all_logits=True)['logits'])
+
+
+def test_packed_checkpoint_with_bias_round_trips(llama, tmp_path):
+    """config.bias = True: the biases of the packed attention projections are parameters, so they are saved and loaded."""
+    from quest_amd import checkpoint
+    torch.manual_seed(9)
+    cfg = llama.LlamaConfig(**{**CFG, 'bias': True})
+    model = llama.Llama(cfg).to(torch.bfloat16).to(DEV).eval()
+    for blk in model.transformer.h:                      # the default initialisation zeroes biases: make them count
+        for lin in (blk.attn.c_attn, blk.attn.c_proj):
+            if lin.bias is not None:
+                torch.nn.init.normal_(lin.bias, std=0.5)
+    llama.quantize_model(model, 'int4', use_hadamard=True, fuse_gate_up=True)
+    packed_biases = [k for k in model.state_dict() if k.endswith('.bias') and '.attn.' in k]
+    assert packed_biases, 'biases must be part of the state dict'
+    path = str(tmp_path / 'mb.safetensors')
+    checkpoint.save_llama(path, model, use_hadamard=True, fuse_gate_up=True)
+    back = checkpoint.load_llama(path, DEV).eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 40), generator=torch.Generator().manual_seed(10)).to(DEV)
+    with torch.no_grad():
+        assert torch.equal(model(ids, all_logits=True)['logits'], back(ids, all_logits=True)['logits'])
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_trained_checkpoint_path_against_fake_quant_model(llama, dtype, capsys):
+    """A checkpoint of the reference's model (parameter names behind its training wrapper's `_orig_mod.module.`
+    prefix, src/eval_hswag.py:187-195) loaded with `load_reference_state_dict`, packed to INT4 and run on the GPU,
+    against the CPU forward whose every linear is the training-side fake-quantised layer (eval_hswag.py:156-217).
+    The packed path rounds the rotated activations to 16 bits before quantising, so some codes sit one level away
+    from the fake-quantised ones, layer after layer; the CPU oracle of the reference's own inference path is at the
+    same distance from the fake-quantised model, which is the bound asserted here (plus an absolute ceiling)."""
+    torch.manual_seed(11)
+    cfg = llama.LlamaConfig(**CFG)
+    donor = llama.Llama(cfg).to(dtype)
+    weights = {k: v.detach().clone() for k, v in donor.state_dict().items()}
+    ckpt = {'_orig_mod.module.' + k: v for k, v in weights.items()}
+    ckpt['_orig_mod.module.transformer.h.0.attn.c_attn.weight_quantizer.scale'] = torch.ones(1)     # ignored extras
+    torch.manual_seed(12)
+    model = llama.Llama(cfg).to(dtype).to(DEV).eval()          # different random weights: the load must replace them
+    llama.load_reference_state_dict(model, ckpt)
+    llama.quantize_model(model, 'int4', use_hadamard=True, fuse_gate_up=True)
+    ids = torch.randint(0, cfg.vocab_size, (2, 32), generator=torch.Generator().manual_seed(13))
+    with torch.no_grad():
+        got = model(ids.to(DEV), all_logits=True)['logits'].double().cpu()
+    fake = lo.forward(weights, ids, cfg.n_layer, cfg.n_head, cfg.rmsnorm_eps, linear='fake_quant').double()
+    w4a4 = lo.forward(weights, ids, cfg.n_layer, cfg.n_head, cfg.rmsnorm_eps, use_hadamard=True).double()
+    dense = lo.forward(weights, ids, cfg.n_layer, cfg.n_head, cfg.rmsnorm_eps, linear='dense').double()
+    err = float((got - fake).norm() / fake.norm())
+    err_ref = float((w4a4 - fake).norm() / fake.norm())
+    gap = float((fake - dense).norm() / dense.norm())
+    with capsys.disabled():
+        print(f'\n[trained-checkpoint path, {dtype}] packed GPU logits vs fake-quant model: {err:.3f}; CPU oracle of the '
+              f'inference path vs fake-quant model: {err_ref:.3f}; fake-quant vs dense model: {gap:.3f}')
+    assert err < 0.25 and err < 1.5 * err_ref + 0.02 and err < gap, (err, err_ref, gap)
