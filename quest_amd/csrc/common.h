@@ -221,6 +221,37 @@ __device__ __forceinline__ int quant_code_inv_i(float x, float inv) {
     asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(m));
     return q;
 }
+// The same code without a clamp instruction, for scales in [2^-99, 2^15] (kQuantFastMin/Max; the caller takes the
+// med3 form above for any other scale, NaN and zero included): t = x * (inv * 2^28), the same nudge, and the
+// floor-and-convert instruction, which saturates at +-2^31; the top four bits of the resulting integer are then the
+// two's-complement nibble of clamp(floor(x / s), -8, 7): floor(floor(2^28 y) / 2^28) = floor(y), and the
+// saturation at +-2^31 is the clamp at -8 and 8 - 2^-28.  (Above 2^15 a quotient of 16-bit floats can underflow
+// fp32 where the product with 2^28 does not; below 2^-99 inv * 2^28 overflows.)
+// `x` must be finite and |x / s| < 2^99, which holds when s is the Gaussian or absmax scale of x's own row.
+__device__ constexpr float kQuantFastMin = 0x1p-99f, kQuantFastMax = 0x1p15f;
+__device__ __forceinline__ bool quant_fast_ok(float s) { return s >= kQuantFastMin && s <= kQuantFastMax; }
+__device__ __forceinline__ float quant_inv28(float s) { return __fmul_rn(__fdiv_rn(1.0f, s), 0x1p28f); }
+__device__ __forceinline__ int quant_top_nibble(float x, float inv28) {
+    const float t = __fmul_rn(x, inv28);
+    const float tn = __builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t);
+    int q;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(tn));
+    return q;
+}
+// ... for any finite or infinite x (a product that overflows to -inf turns the nudge into inf - inf = NaN, which
+// the maximum replaces by the most negative float: code -8, as the clamp of the reference gives)
+__device__ __forceinline__ int quant_top_nibble_any(float x, float inv28) {
+    const float t = __fmul_rn(x, inv28);
+    float tn = __builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t);
+    tn = __builtin_fmaxf(tn, -3.4028234663852886e38f);
+    int q;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(tn));
+    return q;
+}
+// appends the nibble in the top four bits of `n` below the nibbles already in `packed` (which move up by four bits)
+__device__ __forceinline__ uint32_t push_top_nibble(uint32_t packed, int n) {
+    return __builtin_amdgcn_alignbit(packed, (uint32_t)n, 28);
+}
 // reference form with the correctly rounded divide (kept for the exhaustive equivalence test)
 __device__ __forceinline__ float quant_code(float x, float s) {
     float q = __builtin_floorf(__fdiv_rn(x, s));

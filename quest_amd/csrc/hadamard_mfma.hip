@@ -250,7 +250,6 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
         for (int w = 0; w < WPR; w++) total += part_sq[row_local * WPR + w];       // fixed order: every wave gets the same bits
     }
     const uint32_t s16 = from_f32<DT>(scale_from_sumsq(total, K));
-    const float inv = quant_inv(to_f32<DT>(s16));
     const bool writer = lane % G == 0 && h == 0 && part == 0 && row < M;      // one lane per row
 
     if (x_had != nullptr && live) {
@@ -264,31 +263,47 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
     if (writer) scale[row] = (uint16_t)s16;
     if (packed == nullptr && row_sum == nullptr) return;      // uniform over the workgroup
 
-    // ---- codes: c3 c2 c1 c0 (outputs 8 Q + 4 h + {0..3}, Q = 4 mt + q) summed as c_e 16^e: the two's-complement
-    // nibbles once 0x8888 is added (no borrows between offset-binary nibbles) and the top bits are flipped back
-    int hw[16];
+    // ---- codes.  Outputs 8 Q + 4 h + {0..3} (Q = 4 mt + q) give one half-word c3 c2 c1 c0 of two's-complement nibbles.
+    // Scales in the quantiser's fast range (everything but degenerate rows) take the clamp-free form: the code
+    // arrives in the top nibble of an integer and is shifted into the half-word by one v_alignbit per code.
+    const float sf = to_f32<DT>(s16);
+    uint32_t hw[16];
+    if (__builtin_amdgcn_ballot_w64(row < M && !quant_fast_ok(sf)) == 0) {
+        const float inv28 = quant_inv28(sf);
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+        for (int mt = 0; mt < 4; mt++)
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint32_t w0 = yb[mt][q * 2], w1 = yb[mt][q * 2 + 1];
-            const int c0 = quant_code_inv_i(lo_f32<DT>(w0), inv);
-            const int c1 = quant_code_inv_i(hi_f32<DT>(w0), inv);
-            const int c2 = quant_code_inv_i(lo_f32<DT>(w1), inv);
-            const int c3 = quant_code_inv_i(hi_f32<DT>(w1), inv);
-            hw[mt * 4 + q] = ((c3 * 16 + c2) * 16 + c1) * 16 + c0;
-        }
-    // lane (n, 0) ends with dwords 0..7 of the block's 64 packed bytes, lane (n, 1) with dwords 8..15;
-    // every code sits in exactly one lane's dwords, so the row sum is the sum of their signed nibbles
-    const uint32_t perm_sel = h ? 0x03020706u : 0x05040100u;
-    const int partner = (lane ^ 32) * 4;
+            for (int q = 0; q < 4; q++) {
+                const uint32_t w0 = yb[mt][q * 2], w1 = yb[mt][q * 2 + 1];
+                uint32_t g = (uint32_t)quant_top_nibble(hi_f32<DT>(w1), inv28) >> 28;
+                g = push_top_nibble(g, quant_top_nibble(lo_f32<DT>(w1), inv28));
+                g = push_top_nibble(g, quant_top_nibble(hi_f32<DT>(w0), inv28));
+                hw[mt * 4 + q] = push_top_nibble(g, quant_top_nibble(lo_f32<DT>(w0), inv28));
+            }
+    } else {
+        const float inv = quant_inv(sf);
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t w0 = yb[mt][q * 2], w1 = yb[mt][q * 2 + 1];
+                const uint32_t c0 = (uint32_t)quant_code_inv_i(lo_f32<DT>(w0), inv) & 15u;
+                const uint32_t c1 = (uint32_t)quant_code_inv_i(hi_f32<DT>(w0), inv) & 15u;
+                const uint32_t c2 = (uint32_t)quant_code_inv_i(lo_f32<DT>(w1), inv) & 15u;
+                const uint32_t c3 = (uint32_t)quant_code_inv_i(hi_f32<DT>(w1), inv) & 15u;
+                hw[mt * 4 + q] = (((c3 * 16 + c2) * 16 + c1) * 16) + c0;
+            }
+    }
+    // lane (n, 0) ends with dwords 0..7 of the block's 64 packed bytes, lane (n, 1) with dwords 8..15: dword D is the
+    // half-word Q = D of lane (n, 0) below that of lane (n, 1).  v_permlane32_swap hands the lower lane both half-words
+    // t and the upper lane both half-words t + 8.  Every code sits in exactly one lane's dwords, so the row sum is the
+    // sum of their signed nibbles.
     int isum = 0;
     uint32_t dw[8];
 #pragma unroll
     for (int t = 0; t < 8; t++) {
-        const uint32_t own = ((uint32_t)hw[t + 8] << 16) + (uint32_t)hw[t] + 0x88888888u;      // modulo 2^32
-        const uint32_t other = (uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)own);
-        dw[t] = __builtin_amdgcn_perm(other, own, perm_sel) ^ 0x88888888u;
+        const auto sw = __builtin_amdgcn_permlane32_swap(hw[t], hw[t + 8], false, false);
+        dw[t] = sw[0] | (sw[1] << 16);
         isum = __builtin_amdgcn_sdot8((int)dw[t], 0x11111111, isum, false);
     }
     if (packed != nullptr && live) {

@@ -217,12 +217,21 @@ quantize_kernel(uint16_t *__restrict__ x, const uint16_t *__restrict__ scale, in
     const float s = to_f32<DT>(scale[row]);
     const float half_s = __fmul_rn(s, 0.5f);
     const float inv = quant_inv(s);
+    // scales in the fast range take the clamp-free form of the quantiser (in its variant for arbitrary inputs: this
+    // entry point pairs any x with any scale), the others the med3 form; both equal the IEEE-divide statement
+    const bool fast = quant_fast_ok(s);
+    const float inv28 = quant_inv28(s);
     int isum = 0;
     for (int c = threadIdx.x; c < nchunks; c += 256) {
         float v[8], q[8];
         unpack8<DT>(xr[c], v);
+        if (fast) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = quant_code_inv(v[e], inv);
+            for (int e = 0; e < 8; e++) q[e] = (float)(quant_top_nibble_any(v[e], inv28) >> 28);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) q[e] = quant_code_inv(v[e], inv);
+        }
         if (do_dequantize) {
 #pragma unroll
             for (int e = 0; e < 8; e++) v[e] = __fadd_rn(__fmul_rn(q[e], s), half_s);
