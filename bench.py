@@ -33,7 +33,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-REPLAYS = 7                  # timed replays of a batch of launches; the median is reported
+REPLAYS = 9                  # timed replays of a batch of launches; the median is reported
+WARM_REPLAYS = 3             # untimed replays before them: the first ones run while the clocks still ramp
 EAGER_BATCHES = False        # --eager-batches: time plain launches instead of graph replays
 LAST = {'min_ms': None}      # fastest replay of the most recent launches_ms() call
 INT8_MFMA_PEAK_TOPS = 5000.0
@@ -87,7 +88,8 @@ def launches_ms(launch, n, warmup=5):
             for i in range(n):
                 launch(i)
     torch.cuda.current_stream().wait_stream(side)
-    graph.replay()                               # once untimed
+    for _ in range(WARM_REPLAYS):
+        graph.replay()
     per_launch = []
     for _ in range(REPLAYS):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -368,8 +370,18 @@ def bench_small_layer_gpu(quest, dev):
         quest.fused_matmul_dequantize_int4_int4t_bf16(packed, wp, row_sum, wa, scale, ws, out)
 
     ms = launches_ms(layer, 100, 10)
-    return {'ms_per_call': ms, 'value': 2.0 * m * n * k / (ms * 1e-3) / 1e12, 'unit': 'TOPS',
-            'what': 'the same layer through the HIP path on the GPU (graph replay, median of seven)'}
+    # the checker: activation codes of this workload against the full CPU oracle pipeline on the same x (the
+    # reference's F.linear Hadamard, torch-CPU scale, quantiser), and the layer output against the oracle's
+    from oracle import quest_oracle as qo
+    _, o_scale, o_packed, _ = qo.hadamard_quantize_int4(x.cpu(), hadamard='matmul')
+    differ = (qo.unpack_int4(packed.cpu()) != qo.unpack_int4(o_packed)).float().mean().item()
+    owp, ows, owa, _ = qo.preprocess_weight(w.cpu(), use_hadamard=True, w_scale_mode='absmax')
+    want = qo.linear_forward(x.cpu(), owp, ows, owa, use_hadamard=True, hadamard='matmul', via='fp32').double()
+    rel = ((out.cpu().double() - want).norm() / want.norm()).item()
+    return {'ms_per_call': ms, 'activation_codes_differing_from_oracle_pipeline': differ,
+            'weights_bit_exact': bool(torch.equal(wp.cpu(), owp) and torch.equal(wa.cpu(), owa)),
+            'output_rel_error_vs_oracle': rel, 'value': 2.0 * m * n * k / (ms * 1e-3) / 1e12, 'unit': 'TOPS',
+            'what': 'the same layer through the HIP path on the GPU (graph replay, median of nine)'}
 
 
 def bench_cpu_baseline():

@@ -312,8 +312,10 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
             *reinterpret_cast<uint4 *>(dst) = make_uint4(dw[0], dw[1], dw[2], dw[3]);
             *reinterpret_cast<uint4 *>(dst + 4) = make_uint4(dw[4], dw[5], dw[6], dw[7]);
         } else {                                                          // a view that starts 4 bytes into an allocation
+            // (volatile: kept apart from the vector stores above, which the compiler would otherwise merge with these
+            // into a common, narrower sequence)
 #pragma unroll
-            for (int t = 0; t < 8; t++) dst[t] = dw[t];
+            for (int t = 0; t < 8; t++) *reinterpret_cast<volatile uint32_t *>(dst + t) = dw[t];
         }
     }
     if (row_sum != nullptr) {
