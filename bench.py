@@ -142,6 +142,7 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         if ev:
             ev[2].record()
 
+    lib = _lib.load()
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
@@ -181,7 +182,6 @@ def bench_linear(quest, _lib, steps, warmup, dev):
 
     # the GEMM alone, bare C-ABI launches: on uniform random activation codes (the stated GEMM workload; the
     # matrix cores draw the most power on them) and on the codes the last step left (Gaussian activations)
-    lib = _lib.load()
     u_codes = torch.randint(-8, 8, (m, k), generator=g, dtype=torch.int8)
     u_packed = ((u_codes[:, 1::2] << 4) | (u_codes[:, ::2] & 0xF)).view(torch.uint8).to(dev)
     u_row_sum = u_codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32).to(dev)
@@ -196,6 +196,16 @@ def bench_linear(quest, _lib, steps, warmup, dev):
                 raise RuntimeError('GEMM launch failed')
         return gemm
 
+    # the activation kernel of the step alone (fp16 [4096, 4096], inputs rotating): bare launches in a graph, without the
+    # events that quant_ms above has around it
+    q_tail = (_lib.ptr(a_scale), _lib.ptr(a_packed), _lib.ptr(a_row_sum), None, k, m, 181. / 2048., _lib.DTYPE_CODE[dtype])
+    act_ptrs = [_lib.ptr(x) for x in acts]
+
+    def quant_alone(i):
+        if lib.quest_hadamard_quantize_int4(act_ptrs[i % n_buf], *q_tail, current_stream()) != 0:
+            raise RuntimeError('activation kernel launch failed')
+
+    quant_alone_ms = launches_ms(quant_alone, 100)
     gemm_quantized_ms = launches_ms(gemm_launcher(a_packed, a_row_sum, a_scale), max(steps, 100))
     # the same with the weights rotated through 14 copies (315 MB, more than the Infinity Cache holds), as a model
     # with many layers would stream them from HBM
@@ -224,6 +234,7 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         'gemm_quantized_acts_ms': gemm_quantized_ms,
         'gemm_rotating_weights_ms': gemm_rotating_ms,
         'quant_ms': quant_ms,
+        'quant_alone_ms': quant_alone_ms,
     }
 
 
@@ -485,6 +496,10 @@ def main():
         'gemm_tops_on_quantized_activations': 2.0 * 4096 * 4096 * 11008 / (lin['gemm_quantized_acts_ms'] * 1e-3) / 1e12,
         'quantize_us_in_step': lin['quant_ms'] * 1e3,
         'quantize_GBs': rq['achieved'],
+        'quantize_in_step_shape': {'workload': 'fp16 [4096,4096] (the step\'s own activation kernel), graph of 100 bare launches',
+                                   'us_per_launch': lin['quant_alone_ms'] * 1e3,
+                                   'GBs': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9,
+                                   'frac_hbm': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS},
         'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'few_hundred_tokens': few_hundred, 'forward': fwd, 'cpu_baseline': cpu,
     }
     print(json.dumps(line))

@@ -238,6 +238,23 @@ __device__ __forceinline__ int quant_top_nibble(float x, float inv28) {
     asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(tn));
     return q;
 }
+// The same on the low / high half of a dword of two 16-bit floats.  fp16 halves go into the multiplication as they
+// are (v_fma_mix_f32 converts its selected half on the way in; its addend +0 only turns a product of -0 into +0,
+// which the nudge does anyway); bf16 halves are fp32 bit patterns once shifted or masked.
+template <int DT, int HI>
+__device__ __forceinline__ int quant_top_nibble_half(uint32_t w, float inv28) {
+    if constexpr (DT == QUEST_DTYPE_BF16) {
+        return quant_top_nibble(HI ? hi_f32<DT>(w) : lo_f32<DT>(w), inv28);
+    } else {
+        float t;
+        if constexpr (HI) asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(t) : "v"(w), "v"(inv28));
+        else asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(w), "v"(inv28));
+        const float tn = __builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t);
+        int q;
+        asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(tn));
+        return q;
+    }
+}
 // ... for any finite or infinite x (a product that overflows to -inf turns the nudge into inf - inf = NaN, which
 // the maximum replaces by the most negative float: code -8, as the clamp of the reference gives)
 __device__ __forceinline__ int quant_top_nibble_any(float x, float inv28) {

@@ -275,10 +275,10 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const uint32_t w0 = yb[mt][q * 2], w1 = yb[mt][q * 2 + 1];
-                uint32_t g = (uint32_t)quant_top_nibble(hi_f32<DT>(w1), inv28) >> 28;
-                g = push_top_nibble(g, quant_top_nibble(lo_f32<DT>(w1), inv28));
-                g = push_top_nibble(g, quant_top_nibble(hi_f32<DT>(w0), inv28));
-                hw[mt * 4 + q] = push_top_nibble(g, quant_top_nibble(lo_f32<DT>(w0), inv28));
+                uint32_t g = (uint32_t)quant_top_nibble_half<DT, 1>(w1, inv28) >> 28;
+                g = push_top_nibble(g, quant_top_nibble_half<DT, 0>(w1, inv28));
+                g = push_top_nibble(g, quant_top_nibble_half<DT, 1>(w0, inv28));
+                hw[mt * 4 + q] = push_top_nibble(g, quant_top_nibble_half<DT, 0>(w0, inv28));
             }
     } else {
         const float inv = quant_inv(sf);
