@@ -42,6 +42,8 @@ INT8_MFMA_PEAK_TOPS = 5000.0
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
 # scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
+TRAFFIC_SOURCE = ('constant from a separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this script, summarised in '
+                  'profiles/bench_gemm_M4096_K4096_N11008_and_quantize_8192x4096.md; not measured in this run')
 TRAFFIC_GEMM_BYTES = 343050684
 TRAFFIC_QUANTIZE_BYTES = 84238194
 
@@ -283,7 +285,7 @@ def bench_quantize(_lib, steps, warmup, dev):
     del big
     torch.cuda.empty_cache()
     return {'bound': 'hbm', 'achieved': gbs, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs / HBM_PEAK_GBS,
-            'traffic': TRAFFIC_QUANTIZE_BYTES, 'kernel': 'hadamard_quantize_mfma_kernel', 'us_per_launch': ms * 1e3, 'us_per_launch_min': ms_min * 1e3,
+            'traffic': TRAFFIC_QUANTIZE_BYTES, 'traffic_source': TRAFFIC_SOURCE, 'kernel': 'hadamard_quantize_mfma_kernel', 'us_per_launch': ms * 1e3, 'us_per_launch_min': ms_min * 1e3,
             'algorithmic_bytes': algo_bytes, 'workload': 'bf16 [8192,4096] Student-t(3), 1% channels x20',
             'sustained_at_8x_rows': sustained}
 
@@ -448,6 +450,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-forward', action='store_true', help='skip the whole-model row')
+    ap.add_argument('--layer-sweep', action='store_true',
+                    help='also run the layer benchmark of quest_amd.bench_layer (quick set of token counts) and add it to the line')
     ap.add_argument('--eager-batches', action='store_true',
                     help='time batches of plain launches instead of HIP-graph replays (for rocprofv3 --pmc runs)')
     args = ap.parse_args()
@@ -471,13 +475,17 @@ def main():
     dec = bench_decode(_lib, dev)
     few_hundred = bench_decode(_lib, dev, ms=(128, 256, 384))
     fwd = None if args.no_forward else bench_forward(dev)
+    layer_sweep = None
+    if args.layer_sweep:
+        from quest_amd import bench_layer
+        layer_sweep = bench_layer.as_records(bench_layer.get_timing(batch_sizes=[32, 512, 4096, 16384]))
     calibration_stream(dev)
     cpu = None if args.no_cpu_baseline else bench_cpu_baseline()
     if cpu is not None:
         cpu['gpu_same_workload'] = bench_small_layer_gpu(quest, dev)
 
     roofline = {'bound': 'mfma', 'achieved': lin['gemm_tops'], 'peak': INT8_MFMA_PEAK_TOPS, 'unit': 'TOP/s',
-                'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES,
+                'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES, 'traffic_source': TRAFFIC_SOURCE,
                 'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
                 'us_per_launch_min': lin['gemm_min_ms'] * 1e3,
                 'us_per_launch_weights_from_hbm': lin['gemm_rotating_weights_ms'] * 1e3,
@@ -502,6 +510,8 @@ def main():
                                    'frac_hbm': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS},
         'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'few_hundred_tokens': few_hundred, 'forward': fwd, 'cpu_baseline': cpu,
     }
+    if layer_sweep is not None:
+        line['layer_sweep'] = layer_sweep
     print(json.dumps(line))
 
 

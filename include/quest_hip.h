@@ -104,7 +104,16 @@ int quest_hadamard128(void *y, const void *x, int group_size, int batch_size, fl
  * quest_find_scale_int4 on the transformed row), INT4 codes packed (as quest_quantize_int4) and
  * their row sums.  x is read once and never written.  x_had, when not NULL, receives the
  * transformed activations (dtype) the scale and codes were computed from.  scale is required;
- * x_int_packed and x_int_row_sum are optional.  group_size % 128 == 0, group_size <= 65536.
+ * x_int_packed and x_int_row_sum are optional.  group_size % 128 == 0 and <= 65536 (had_scale == 0:
+ * group_size % 8 == 0, every K the GEMM takes).
+ * Which arithmetic runs depends on (group_size, had_scale, dtype) only, never on batch_size or on where the buffers
+ * lie: a had_scale the dtype holds exactly (181/2048) with group_size <= 32768 is the product with the +-had_scale
+ * matrix on the matrix cores, fp32 accumulation, as the reference states the activation transform; any other factor
+ * (2^-3.5, the weight-side one), and rows over 32768, are fp32 butterflies followed by one multiplication.  The two
+ * agree to fp32 summation noise (<= 1e-3 relative, the transform's stated bar), so that a value on a rounding boundary
+ * of the dtype may come out one ulp apart and its code one level apart: codes are reproducible for a given shape,
+ * factor and dtype, not across the two.  Given the transformed tensor and the scale, codes and row sums are exactly
+ * quest_quantize_int4's in both.
  */
 int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t *x_int_packed,
                                  int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size,
