@@ -450,6 +450,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-forward', action='store_true', help='skip the whole-model row')
+    ap.add_argument('--only', choices=('quantize', 'decode'),
+                    help='run one leg only and print its result (for short rocprofv3 runs): the activation kernel or the decode shapes')
     ap.add_argument('--layer-sweep', action='store_true',
                     help='also run the layer benchmark of quest_amd.bench_layer (quick set of token counts) and add it to the line')
     ap.add_argument('--eager-batches', action='store_true',
@@ -468,6 +470,12 @@ def main():
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
 
+    if args.only == 'quantize':
+        print(json.dumps({'roofline_quantize': bench_quantize(_lib, max(args.steps, 100), args.warmup, dev)}))
+        return
+    if args.only == 'decode':
+        print(json.dumps({'decode': bench_decode(_lib, dev)}))
+        return
     # the bandwidth-bound kernel first: after a few hundred GEMM launches the power controller holds the core clock
     # down for a while, which this kernel (a third of its time is arithmetic) would inherit
     rq = bench_quantize(_lib, max(args.steps, 100), args.warmup, dev)
