@@ -100,8 +100,12 @@ def _gemm_inputs(m, k, n, seed, dtype=torch.float16):
     return a, b, pack(a), pack(b), a_add, b_add, a_mul, b_mul
 
 
-def test_prefill_gemm_4096x4096x11008(quest):
-    m, k, n = 4096, 4096, 11008
+# the prefill shape of the benchmark (the XCD groups divide the channels); the model's QKV and MLP-output shapes at
+# 32 x 512 tokens (more tokens than channels: the groups divide the token tiles), one in each tile shape; a token
+# count that leaves the groups unequal shares of token tiles
+@pytest.mark.parametrize('shape', [(4096, 4096, 11008), (16384, 1024, 3072), (16384, 2816, 1024), (9000, 512, 4104)])
+def test_prefill_gemm_full_size(quest, shape):
+    m, k, n = shape
     a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=0)
     gap, gbp = ap.to(DEV), bp.to(DEV)
     c = quest.matmul_int4_int4t_int32(gap, gbp)
