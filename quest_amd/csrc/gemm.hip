@@ -1193,12 +1193,14 @@ static int gemm_launch_big(void *out, const uint8_t *a, const uint8_t *b, const 
 // as one round of 128 x 128 tiles (half the operand bytes per MFMA) is 15-20 % faster.  Measured against the other
 // kernels over M from 65 to 4096 with (K, N) from (1024, 3072) to (8192, 8192): 1.2 to 2.6 x faster where this picks
 // small tiles.
-// Up to 64 tokens the weight-streaming kernel is the faster one while there are few channels or one token tile; with
-// thousands of channels and more than one (two at N = 8192) of its 16-token tiles, one small tile of 64 tokens per
-// 64 channels is up to 2 x faster (measured at N from 8192 to 28672).
+// Up to 64 tokens the weight-streaming kernel is the faster one while its N / 16 workgroups are one per CU or fewer, or
+// it has one or two token tiles; beyond that its time grows with its token tiles: 33 to 64 tokens (four tiles) take one
+// small tile of 64 tokens per 64 channels from N > 4096 on (measured at N = 4608 .. 11264, K = 2048 and 4096: 8.3 -> 5.4 us,
+// 11.2 -> 7.6 us; at N = 4096 the weight-streaming kernel is 0.6 to 1.2 us faster), 17 to 32 tokens from N > 8192 on (up to
+// 2 x faster at N from 8192 to 28672).
 static int small_tile_shape(int M, int K, int N, int cus) {
     if ((K & 255) != 0) return 0;
-    if (M <= 64) return (M > 16 && N >= 8192 && (M > 32 || N > 8192)) ? 64 : 0;
+    if (M <= 64) return (M > 32 ? N > 4096 : (M > 16 && N > 8192)) ? 64 : 0;
     const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
     const long per_cu = (tiles + cus - 1) / cus;
     if (per_cu <= 3) return 64;
