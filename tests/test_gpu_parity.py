@@ -150,7 +150,7 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048), (66, 4096, 8),
                (640, 2816, 1024),
                # ... and a few tens of tokens with thousands of channels
-               (40, 256, 8200), (64, 512, 11008), (17, 256, 11010), (33, 256, 8192),
+               (40, 256, 8200), (64, 512, 11008), (17, 256, 11010), (33, 256, 8192), (48, 512, 4610), (64, 256, 4096),
                # four 64 x 64 tiles per CU = one round of 128 x 128 tiles (ragged in both directions); one tile per
                # workgroup of the large-tile kernel, cut along single token tiles
                (1000, 512, 4090), (1536, 256, 4096), (768, 128, 8200), (1300, 384, 4100),
@@ -190,7 +190,7 @@ def test_matmul_int32_extreme_codes(quest):
                                    (4096, 256, 2048), (16384, 128, 2048),
                                    # a few hundred tokens, K % 256 == 0 (small tiles): ragged tiles, vector and element-wise stores
                                    (127, 512, 33), (130, 256, 1000), (448, 768, 4100), (70, 1024, 4097), (1000, 512, 2048),
-                                   (66, 4096, 8), (640, 2816, 1024), (40, 256, 8200), (64, 512, 11008), (17, 256, 11010),
+                                   (66, 4096, 8), (640, 2816, 1024), (40, 256, 8200), (64, 512, 11008), (17, 256, 11010), (48, 512, 4610),
                                    (1000, 512, 4090), (1536, 256, 4096), (768, 128, 8200), (1300, 384, 4100),
                                    # odd token and channel counts in the large-tile kernel
                                    (301, 384, 512), (1001, 128, 96), (4097, 128, 1031), (777, 1152, 4100),
