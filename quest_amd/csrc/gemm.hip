@@ -1221,8 +1221,8 @@ static int gemm_launch_small(void *out, const uint8_t *a, const uint8_t *b, cons
 
 // Wide (256 x 256 tiles, a lone wave per SIMD) has the cheaper main loop; Duo (256 x 128, two workgroups per CU)
 // hides epilogues and waits.  Duo wins where there is enough work for full-width tiles on 512 workgroups (256 cells
-// of 256 tokens x 32 channels per XCD group) and the epilogue weighs much: K short, or fewer than 16 channel units
-// per group, which would leave Wide with narrow tiles.  Measured over M in {1024, 4096, 16384}, K in {1024 .. 11008},
+// of 256 tokens x 32 channels per XCD group) and the epilogue weighs much: K short, or at most 16 channel units
+// per group (N <= 4096), which would leave Wide with narrow tiles.  Measured over M in {1024, 4096, 16384}, K in {1024 .. 11008},
 // N in {1024 .. 11008} (and again over M from 512): in total run time the rule is within 0.3 % of always picking the
 // faster shape, and within 7 % on every single size.
 template <int OUT, bool GLU>
@@ -1236,7 +1236,7 @@ static int gemm_launch_large(void *out, const uint8_t *a, const uint8_t *b, cons
     const long cells_per_group = (long)((M + big::kRows - 1) / big::kRows) * per_group;
     // small problems (fewer cells per group than Wide has workgroups): twice the workgroups help while K is short
     const bool small = cells_per_group <= 32 && K <= (cells_per_group <= 24 ? 4096 : 2816);
-    const bool duo = small || (cells_per_group >= 256 && (K <= 1024 || per_group < 16));
+    const bool duo = small || (cells_per_group >= 256 && (K <= 1024 || per_group <= 16));
     if (!duo) return gemm_launch_big<big::Wide, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     return gemm_launch_big<big::Duo, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
 }
