@@ -45,8 +45,8 @@ INT8_MFMA_PEAK_TOPS = 5000.0
 # the runs are summarised under profiles/.
 TRAFFIC_SOURCE = ('constant from a separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this script, summarised in '
                   'profiles/bench_gemm_M4096_K4096_N11008_and_quantize_8192x4096.md; not measured in this run')
-TRAFFIC_GEMM_BYTES = 343106784
-TRAFFIC_QUANTIZE_BYTES = 84235068
+TRAFFIC_GEMM_BYTES = 343078377
+TRAFFIC_QUANTIZE_BYTES = 84236564
 
 
 def event_pairs(n):
