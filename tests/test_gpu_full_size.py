@@ -88,6 +88,28 @@ def test_activation_kernel_8192x4096(quest):
     assert torch.equal(row_sum[rows.to(DEV)].cpu(), want_sum)
 
 
+def test_activation_tensor_of_2_gib_and_more(quest):
+    """An input of 2 GiB and more goes to the kernel as several launches of whole rows (32-bit offsets inside one):
+    the rows either side of the cut, the first and the last ones must equal what the same rows give as a tensor of
+    their own, bit for bit, and every row sum must match its codes."""
+    k = 4096
+    cut = ((1 << 31) - 1) // (2 * k)                 # rows in the first launch: 262143
+    m = cut + 300
+    g = torch.Generator(device=DEV).manual_seed(5)
+    x = torch.randn(m, k, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    assert x.numel() * 2 >= 1 << 31
+    scale, packed, row_sum = quest.hadamard_quantize_int4(x)
+    for lo, hi in ((0, 128), (cut - 160, cut + 160), (m - 128, m)):
+        s2, p2, r2 = quest.hadamard_quantize_int4(x[lo:hi])
+        assert torch.equal(bits(scale[lo:hi].cpu()), bits(s2.cpu())), (lo, hi)
+        assert torch.equal(packed[lo:hi], p2) and torch.equal(row_sum[lo:hi], r2), (lo, hi)
+    step = 32768
+    for lo in range(0, m, step):                      # in pieces: the unpacked codes of everything would be 2 GiB more
+        codes = unpack_gpu(packed[lo:lo + step])
+        assert torch.equal(codes.to(torch.int32).sum(-1, keepdim=True), row_sum[lo:lo + step].to(torch.int32)), lo
+    assert (scale.float() > 0).all()
+
+
 def _gemm_inputs(m, k, n, seed, dtype=torch.float16):
     g = torch.Generator().manual_seed(seed)
     a = torch.randint(-8, 8, (m, k), generator=g, dtype=torch.int8)
