@@ -447,7 +447,27 @@ def bench_cpu_baseline():
         t32.append(time.perf_counter() - t0)
     t32.sort()
     ops = 2.0 * m * n * k
+    # the bench step's own workload (fp16 [4096,4096] -> quantise -> x [11008,4096]^T, same generators as the GPU step):
+    # a warm-up on 256 tokens, then five whole steps, their median counted -- about ten seconds of CPU work
+    sm, sk, sn = 4096, 4096, 11008
+    g = torch.Generator(device='cpu').manual_seed(0)
+    sx = torch.randn(sm, sk, generator=g).half()
+    s_codes = torch.randint(-8, 8, (sn, sk), generator=g, dtype=torch.int8)
+    s_packed = ((s_codes[:, 1::2] << 4) | (s_codes[:, ::2] & 0xF)).view(torch.uint8)
+    s_scale = (torch.rand(sn, 1, generator=g) * 0.09 + 0.01).half()
+    s_add = (s_codes.to(torch.int32).sum(-1, keepdim=True) + sk // 2).to(torch.int32)
+    del s_codes
+    qo.linear_forward(sx[:256], s_packed, s_scale, s_add, use_hadamard=True, hadamard='matmul', via='fp64')
+    t_step = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        qo.linear_forward(sx, s_packed, s_scale, s_add, use_hadamard=True, hadamard='matmul', via='fp64')
+        t_step.append(time.perf_counter() - t0)
+    step_workload = {'what': f'one bench step on the CPU: W4A4 linear fp16 M={sm} K={sk} N={sn}, median of five calls',
+                     's_per_step': sorted(t_step)[2], 'value': 2.0 * sm * sn * sk / sorted(t_step)[2] / 1e12, 'unit': 'TOPS'}
+    del sx, s_packed
     return {'value': ops / med / 1e12, 'unit': 'TOPS', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'step_workload': step_workload,
             'sample': f'W4A4 linear fp16 M={m} K={k} N={n}, seed 0, median of 10 calls after 3 warm-ups '
                       f'({med * 1e3:.1f} ms per call; integer GEMM via fp64 matmul as the reference checks it)',
             'ms_per_call': med * 1e3,
