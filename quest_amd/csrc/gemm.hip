@@ -59,8 +59,9 @@ static int small_tile_shape(int M, int K, int N, int cus) {
 // N in {1024 .. 11008} (and again over M from 512): in total run time the rule is within 0.3 % of always picking the
 // faster shape, and within 7 % on every single size.
 static int gemm_launch_large(int out_kind, bool glu, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
-                             const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    const int small_shape = small_tile_shape(M, K, N, device_cu_count(st));
+                             const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus,
+                             hipStream_t st) {
+    const int small_shape = small_tile_shape(M, K, N, cus);
     if (small_shape != 0) return launch_gemm_small(out_kind, glu, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     const int units = (N + 31) / 32;
     const int per_group = units >= 8 ? units / 8 : units;
@@ -68,12 +69,14 @@ static int gemm_launch_large(int out_kind, bool glu, void *out, const uint8_t *a
     // small problems (fewer cells per group than Wide has workgroups): twice the workgroups help while K is short
     const bool small = cells_per_group <= 32 && K <= (cells_per_group <= 24 ? 4096 : 2816);
     const bool duo = small || (cells_per_group >= 256 && (K <= 1024 || per_group <= 16));
-    return launch_gemm_big(out_kind, glu, duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    return launch_gemm_big(out_kind, glu, duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
 }
 
 static int gemm_launch(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    const int small_shape = small_tile_shape(M, K, N, device_cu_count(st));
+    // the device is asked for its CU count once per call, and only where a rule below uses it (not for a handful of tokens)
+    const int cus = M > 64 ? device_cu_count(st) : 0;
+    const int small_shape = small_tile_shape(M, K, N, cus);
     if (small_shape != 0) return launch_gemm_small(out_kind, false, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     // a handful of tokens: the weight-streaming kernel
     // (up to 64 of them unless the small tiles took the call above; where K rules those out, up to 128 while its
@@ -84,7 +87,7 @@ static int gemm_launch(int out_kind, void *out, const uint8_t *a, const uint8_t 
     }
     // the large-tile kernel fetches the 16-bit scale vectors two per dword: 4-byte aligned vectors
     if ((K & 127) == 0 && M > 64 && aligned(b_mul, 4) && aligned(a_mul, 4))
-        return gemm_launch_large(out_kind, false, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        return gemm_launch_large(out_kind, false, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
     // K % 128 != 0, or scale vectors at odd element offsets (a sliced tensor): the register-staged kernel reads them
     // element by element
     return launch_gemm_staged(out_kind, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
@@ -128,5 +131,6 @@ extern "C" int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, cons
         !aligned(mat_d, 8))
         return QUEST_ERR_UNSUPPORTED;
     return gemm_launch_large(dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16, true, mat_d, mat_a, mat_b, vec_a_add, vec_b_add,
-                             vec_a_mul, vec_b_mul, size_m, size_k, size_n, (hipStream_t)stream);
+                             vec_a_mul, vec_b_mul, size_m, size_k, size_n, device_cu_count((hipStream_t)stream),
+                             (hipStream_t)stream);
 }

@@ -624,12 +624,12 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
 
 template <typename C, int OUT, bool GLU>
 static int launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                           const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+                           const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
     Schedule sch;
     sch.tiles_t = (M + big::kRows - 1) / big::kRows;
     sch.units = (N + 31) / 32;
     const long cells = (long)sch.tiles_t * sch.units;
-    long grid = (long)C::kWgPerCu * device_cu_count(st);      // persistent: one or two workgroups per CU
+    long grid = (long)C::kWgPerCu * cus;                      // persistent: one or two workgroups per CU
     if (grid > cells) grid = cells;
     sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
     sch.row_tiles = 0;
@@ -663,22 +663,22 @@ static int launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32
 
 template <int OUT, bool GLU>
 static int launch_shape(bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    if (duo) return launch_big<big::Duo, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    return launch_big<big::Wide, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+                        const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
+    if (duo) return launch_big<big::Duo, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
+    return launch_big<big::Wide, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
 }
 
 int launch_gemm_big(int out_kind, bool glu, bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
-                    const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    if ((K & 127) != 0 || (glu && out_kind == OUT_INT32)) return QUEST_ERR_UNSUPPORTED;
+                    const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
+    if ((K & 127) != 0 || cus <= 0 || (glu && out_kind == OUT_INT32)) return QUEST_ERR_UNSUPPORTED;
     if (glu) {
-        if (out_kind == OUT_BF16) return launch_shape<OUT_BF16, true>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        return launch_shape<OUT_FP16, true>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        if (out_kind == OUT_BF16) return launch_shape<OUT_BF16, true>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
+        return launch_shape<OUT_FP16, true>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
     }
     switch (out_kind) {
-        case OUT_BF16: return launch_shape<OUT_BF16, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        case OUT_FP16: return launch_shape<OUT_FP16, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        default: return launch_shape<OUT_INT32, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+        case OUT_BF16: return launch_shape<OUT_BF16, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
+        case OUT_FP16: return launch_shape<OUT_FP16, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
+        default: return launch_shape<OUT_INT32, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
     }
 }
 

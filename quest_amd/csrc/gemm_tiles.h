@@ -41,8 +41,8 @@ __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
     }
 }
 
-// Compute units of the device the stream belongs to.  Asked for at every launch (two host-side queries, no stream
-// operation, nothing cached): the library keeps no state and a process may drive several devices.
+// Compute units of the device the stream belongs to.  Asked for once per call that needs it (two host-side queries,
+// no stream operation, nothing cached): the library keeps no state and a process may drive several devices.
 inline int device_cu_count(hipStream_t st) {
     int dev = 0, cus = 0;
     if (hipStreamGetDevice(st, &dev) != hipSuccess && hipGetDevice(&dev) != hipSuccess) return 256;
@@ -51,9 +51,10 @@ inline int device_cu_count(hipStream_t st) {
 }
 
 // gemm_big.hip: the large-tile kernel (K % 128 == 0, 4-byte aligned scale vectors); `duo` picks two workgroups of
-// 256 x 128 tiles per CU instead of one of 256 x 256, `glu` the SwiGLU epilogue (16-bit outputs only)
+// 256 x 128 tiles per CU instead of one of 256 x 256, `glu` the SwiGLU epilogue (16-bit outputs only), `cus` the
+// device's CU count (the persistent grid's size)
 int launch_gemm_big(int out_kind, bool glu, bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
-                    const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);
+                    const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st);
 // gemm_small.hip: tiles of `shape` x `shape` (64 or 128), K % 256 == 0
 int launch_gemm_small(int out_kind, bool glu, int shape, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                       const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);
