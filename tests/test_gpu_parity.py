@@ -114,7 +114,7 @@ def test_quantize_every_16bit_input(quest, dtype):
 
 # --------------------------------------------------------------------------- E1
 @pytest.mark.parametrize('dtype', DTYPES)
-@pytest.mark.parametrize('shape', [(160, 224), (1, 1), (7, 513), (33, 4096)])
+@pytest.mark.parametrize('shape', [(160, 224), (1, 1), (7, 513), (33, 4096), (300, 2056), (5, 8)])
 def test_add_mul_vv(quest, dtype, shape):
     m, n = shape
     g = torch.Generator().manual_seed(3)
@@ -125,6 +125,20 @@ def test_add_mul_vv(quest, dtype, shape):
     b_mul = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype)
     want = qo.add_mul_vv(a_add, a_mul, b_add, b_mul, c)
     got = quest.add_mul_vv(a_add.to(DEV), a_mul.to(DEV), b_add.to(DEV), b_mul.to(DEV), c.to(DEV)).cpu()
+    assert torch.equal(bits(got), bits(want))
+
+
+def test_add_mul_vv_vectors_at_odd_offsets(quest):
+    """Rows of whole eights take 16-byte vector accesses; channel vectors that start at an odd element must not."""
+    m, n = 37, 264
+    g = torch.Generator().manual_seed(4)
+    c = torch.randint(-200000, 200000, (m, n), generator=g, dtype=torch.int32)
+    a_add = torch.randint(-30000, 30000, (m, 1), generator=g, dtype=torch.int32)
+    b_add = torch.randint(-30000, 30000, (n + 1, 1), generator=g, dtype=torch.int32)
+    a_mul = (torch.rand(m, 1, generator=g) * 0.09 + 0.01).to(torch.float16)
+    b_mul = (torch.rand(n + 1, 1, generator=g) * 0.09 + 0.01).to(torch.float16)
+    want = qo.add_mul_vv(a_add, a_mul, b_add[1:], b_mul[1:], c)
+    got = quest.add_mul_vv(a_add.to(DEV), a_mul.to(DEV), b_add.to(DEV)[1:], b_mul.to(DEV)[1:], c.to(DEV)).cpu()
     assert torch.equal(bits(got), bits(want))
 
 
