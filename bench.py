@@ -256,6 +256,16 @@ def bench_linear(quest, _lib, steps, warmup, dev):
     del w_copies
     gemm_ms = launches_ms(gemm_launcher(u_packed, u_row_sum, u_scale), max(steps, 100))
     gemm_min_ms = LAST['min_ms']
+    # a yardstick, not part of the path: the vendor library's INT8 GEMM (torch._int_mm -> hipBLASLt) on the same codes as
+    # int8, int32 out -- twice the operand bytes, no nibbles to split, no scale arithmetic
+    vendor_int8_ms = None
+    try:
+        w8 = w_codes.to(dev)
+        u8 = u_codes.to(dev)
+        vendor_int8_ms = launches_ms(lambda _: torch._int_mm(u8, w8.t()), 50)
+        del w8, u8
+    except Exception:                       # not every build of the library has it
+        vendor_int8_ms = None
     ops = 2.0 * m * n * k
     return {
         'shape': {'M': m, 'K': k, 'N': n},
@@ -270,6 +280,7 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         'gemm_in_step_ms': gemm_in_step_ms,
         'gemm_quantized_acts_ms': gemm_quantized_ms,
         'gemm_rotating_weights_ms': gemm_rotating_ms,
+        'vendor_int8_ms': vendor_int8_ms,
         'quant_ms': quant_ms,
         'quant_alone_ms': quant_alone_ms,
     }
@@ -553,6 +564,7 @@ def main():
                 'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
                 'us_per_launch_min': lin['gemm_min_ms'] * 1e3,
                 'us_per_launch_weights_from_hbm': lin['gemm_rotating_weights_ms'] * 1e3,
+                'vendor_int8_gemm_same_shape_us': None if lin['vendor_int8_ms'] is None else lin['vendor_int8_ms'] * 1e3,
                 'algorithmic_ops': 2.0 * 4096 * 4096 * 11008,
                 'workload': 'uniform random INT4 codes on both sides, M=4096 K=4096 N=11008, fp16 out'}
     line = {
