@@ -222,30 +222,41 @@ quantize_kernel(uint16_t *__restrict__ x, const uint16_t *__restrict__ scale, in
     const bool fast = quant_fast_ok(s);
     const float inv28 = quant_inv28(s);
     int isum = 0;
-    for (int c = threadIdx.x; c < nchunks; c += 256) {
-        float v[8], q[8];
-        unpack8<DT>(xr[c], v);
-        if (fast) {
+    // two chunks per thread and pass, both loads issued before either is used (a row of 4096 is exactly one pass)
+    for (int c0 = threadIdx.x; c0 < nchunks; c0 += 512) {
+        const int c1 = c0 + 256;
+        const bool two = c1 < nchunks;
+        uint4 raw[2];
+        raw[0] = xr[c0];
+        raw[1] = two ? xr[c1] : make_uint4(0, 0, 0, 0);
 #pragma unroll
-            for (int e = 0; e < 8; e++) q[e] = (float)(quant_top_nibble_any(v[e], inv28) >> 28);
-        } else {
+        for (int u = 0; u < 2; u++) {
+            if (u == 1 && !two) break;
+            const int c = u == 0 ? c0 : c1;
+            float v[8], q[8];
+            unpack8<DT>(raw[u], v);
+            if (fast) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) q[e] = quant_code_inv(v[e], inv);
-        }
-        if (do_dequantize) {
+                for (int e = 0; e < 8; e++) q[e] = (float)(quant_top_nibble_any(v[e], inv28) >> 28);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = __fadd_rn(__fmul_rn(q[e], s), half_s);
-            xr[c] = pack8<DT>(v);
-        }
-        const uint32_t w = pack_nibbles8(q, isum);
-        if (packed != nullptr) packed[(size_t)row * nchunks + c] = w;
-        if (x_int != nullptr) {
-            uint2 b;
-            b.x = ((uint32_t)(int)q[0] & 0xFFu) | (((uint32_t)(int)q[1] & 0xFFu) << 8) |
-                  (((uint32_t)(int)q[2] & 0xFFu) << 16) | (((uint32_t)(int)q[3] & 0xFFu) << 24);
-            b.y = ((uint32_t)(int)q[4] & 0xFFu) | (((uint32_t)(int)q[5] & 0xFFu) << 8) |
-                  (((uint32_t)(int)q[6] & 0xFFu) << 16) | (((uint32_t)(int)q[7] & 0xFFu) << 24);
-            reinterpret_cast<uint2 *>(x_int + (size_t)row * K)[c] = b;
+                for (int e = 0; e < 8; e++) q[e] = quant_code_inv(v[e], inv);
+            }
+            if (do_dequantize) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = __fadd_rn(__fmul_rn(q[e], s), half_s);
+                xr[c] = pack8<DT>(v);
+            }
+            const uint32_t w = pack_nibbles8(q, isum);
+            if (packed != nullptr) packed[(size_t)row * nchunks + c] = w;
+            if (x_int != nullptr) {
+                uint2 b;
+                b.x = ((uint32_t)(int)q[0] & 0xFFu) | (((uint32_t)(int)q[1] & 0xFFu) << 8) |
+                      (((uint32_t)(int)q[2] & 0xFFu) << 16) | (((uint32_t)(int)q[3] & 0xFFu) << 24);
+                b.y = ((uint32_t)(int)q[4] & 0xFFu) | (((uint32_t)(int)q[5] & 0xFFu) << 8) |
+                      (((uint32_t)(int)q[6] & 0xFFu) << 16) | (((uint32_t)(int)q[7] & 0xFFu) << 24);
+                reinterpret_cast<uint2 *>(x_int + (size_t)row * K)[c] = b;
+            }
         }
     }
     if (row_sum != nullptr) {
