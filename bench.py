@@ -307,6 +307,14 @@ def bench_quantize(_lib, steps, warmup, dev):
     algo_bytes = m * k * 2 + m * k // 2 + m * 2 + m * 4
     gbs = algo_bytes / (ms * 1e-3) / 1e9
 
+    # a yardstick: torch's device copy moving the same number of bytes in one launch (half read, half written), inputs
+    # rotating as above
+    half = algo_bytes // 2 // 16 * 16
+    flat = [x.view(torch.uint8).view(-1) for x in xs]
+    sink = torch.empty(half, dtype=torch.uint8, device=dev)
+    copy_same_bytes_ms = launches_ms(lambda i: sink.copy_(flat[i % n_buf][:half]), steps, warmup)
+    del flat, sink
+
     # the same kernel on eight times the rows: what it sustains once launch, fill and drain (about 4 us, a fifth of
     # the 8192-row launch) are amortised, next to a device copy of the same size class
     del xs
@@ -333,6 +341,7 @@ def bench_quantize(_lib, steps, warmup, dev):
     return {'bound': 'hbm', 'achieved': gbs, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': gbs / HBM_PEAK_GBS,
             'traffic': TRAFFIC_QUANTIZE_BYTES, 'traffic_source': TRAFFIC_SOURCE, 'kernel': 'hadamard_quantize_mfma_kernel', 'us_per_launch': ms * 1e3, 'us_per_launch_min': ms_min * 1e3,
             'us_per_launch_after_60ms_of_replays': None if ms_sustained is None else ms_sustained * 1e3,
+            'device_copy_same_bytes_us': copy_same_bytes_ms * 1e3,
             'algorithmic_bytes': algo_bytes, 'workload': 'bf16 [8192,4096] Student-t(3), 1% channels x20',
             'sustained_at_8x_rows': sustained}
 
