@@ -163,7 +163,7 @@ def test_prefill_gemm_full_size(quest, shape):
 
 
 @pytest.mark.parametrize('m', [1, 8, 16])
-@pytest.mark.parametrize('kn', [(4096, 4096), (11008, 4096)])
+@pytest.mark.parametrize('kn', [(4096, 4096), (11008, 4096), (4096, 11008)])
 def test_decode_gemm_full_shapes(quest, m, kn):
     k, n = kn
     a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=3 + m)

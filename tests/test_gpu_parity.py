@@ -153,6 +153,8 @@ GEMM_SHAPES = [(160, 768, 224), (1, 4096, 4096), (8, 256, 33), (16, 11008, 512),
                # a handful of tokens (the weight-streaming kernel): 64-byte row tails, ragged N, each token-tile count
                (3, 384, 18), (16, 128, 16), (17, 1152, 64), (32, 640, 100), (40, 2304, 47), (64, 8192, 32), (5, 28672, 24),
                (12, 160, 40), (65, 256, 48), (100, 1152, 300), (128, 4096, 512), (127, 384, 33),
+               # ... 8 to 16 tokens on wide layers: ragged channel counts, the 64-byte row tail
+               (16, 256, 8200), (8, 1152, 11008), (13, 128, 8209), (9, 384, 8193), (7, 256, 8200), (16, 256, 8191),
                # enough cells for the two-workgroups-per-CU shape of the large-tile kernel (>= 256 cells of 256 tokens x
                # 32 channels per XCD group): few channels with a ragged last token tile; short K with a channel count
                # that takes the element-wise epilogue
