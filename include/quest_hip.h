@@ -193,6 +193,43 @@ int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *scale, uint
 int quest_rope_interleaved(void *x, const float *freqs_cis, int n_rows, int seq_len, int row_stride,
                            int rot_cols, int head_dim, int dtype, void *stream);
 
+/*
+ * ---- the FP6 matrix-core path: operands in "E2M3 tiles" ----------------------------------------------------------
+ * Both operands of the reference's fused GEMM are dequantised as (q + 1/2) * scale (quest/quantize_kernel.cu:162,
+ * benchmarks/utils.py:667-678), so 2 C + a_add + b_add of its epilogue (benchmarks/utils.py:544) is
+ * 2 * sum_k (qa + 1/2)(qb + 1/2).  The sixteen values q + 1/2 are exact in FP6 E2M3 and every partial sum of up to
+ * 65536 of their products is exact in fp32, so the gfx950 FP6 matrix instructions (twice the INT8 rate) give the
+ * reference's outputs bit for bit.  These entry points have no counterpart in the reference's quest_c extension;
+ * they are what quest_fused_matmul_dequantize_int4_int4t and quest_hadamard_quantize_int4 are for a caller that keeps
+ * its codes in the operand form instead of packed nibbles.
+ *
+ * E2M3 tiles of a (rows, size_k) code matrix, size_k % 64 == 0: ceil(rows / 32) row blocks x size_k / 64 fragments
+ * of 1536 bytes, row block major.  In fragment (rb, ks), lane l = 32 g + i (row 32 rb + i, codes k = 64 ks + 32 g ..
+ * + 31) owns 32 x 6 bits, code j (the E2M3 bits of q + 1/2) at bits [6 j, 6 j + 6) of its 24 bytes: bytes 0 .. 15 at
+ * fragment offset 16 l, bytes 16 .. 23 at offset 1024 + 8 l.  Rows past `rows` in the last row block hold zeros.
+ */
+
+/* Bytes of the E2M3 tiles of a (rows, size_k) code matrix; 0 for an invalid shape. */
+size_t quest_e2m3_tiles_bytes(int rows, int size_k);
+
+/* tiles = the E2M3 tiles of the packed INT4 codes x_int_packed (rows, size_k / 2), low nibble = even k. */
+int quest_int4_to_e2m3_tiles(void *tiles, const uint8_t *x_int_packed, int rows, int size_k, void *stream);
+
+/*
+ * mat_d (size_m, size_n) dtype = quest_fused_matmul_dequantize_int4_int4t's result for the same codes, from their
+ * E2M3 tiles: dtype( f32(2 S) * (0.5f * vec_a_mul[m] * vec_b_mul[n]) ) with S = sum_k (qa + 1/2)(qb + 1/2) accumulated
+ * exactly.  size_k % 128 == 0 and <= 65536; any size_m, size_n >= 1; scale vectors 4-byte aligned.
+ */
+int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles, const void *vec_a_mul,
+                                       const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
+                                       void *stream);
+
+/* The same with the SwiGLU epilogue of quest_fused_matmul_dequantize_swiglu_int4_int4t (b_tiles and vec_b_mul in its
+ * interleaved row order); mat_d is (size_m, size_n / 2). */
+int quest_fused_matmul_dequantize_swiglu_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles,
+                                              const void *vec_a_mul, const void *vec_b_mul, int size_m, int size_k,
+                                              int size_n, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -233,6 +233,75 @@ def linear_fp64(a_int, a_scale, w_int, w_scale):
 
 
 # ---------------------------------------------------------------------------------------------
+# The FP6 (E2M3) operand form of the codes.  No counterpart in the reference: it is this build's storage format for
+# the codes of the same GEMM, so what the oracle states is the OCP Microscaling FP6 E2M3 number format itself (1 sign
+# bit, 2 exponent bits with bias 1, 3 mantissa bits, subnormals, no Inf/NaN) and the tile layout declared in
+# include/quest_hip.h; tests/test_oracle_pins.py pins the decoder by the format's published value table.
+# ---------------------------------------------------------------------------------------------
+E2M3_FRAGMENT_BYTES = 1536
+
+
+def e2m3_value(bits: torch.Tensor) -> torch.Tensor:
+    """fp64 value of 6-bit E2M3 patterns: (-1)^s * 2^(e-1) * (1 + m/8) for e > 0, (-1)^s * m/8 for e = 0."""
+    bits = bits.to(torch.int64)
+    sign = 1. - 2. * ((bits >> 5) & 1).to(torch.float64)
+    e = (bits >> 3) & 3
+    m = (bits & 7).to(torch.float64)
+    mag = torch.where(e == 0, m / 8., (1. + m / 8.) * torch.pow(torch.tensor(2., dtype=torch.float64), (e - 1).to(torch.float64)))
+    return sign * mag
+
+
+def e2m3_bits_of_code(q: torch.Tensor) -> torch.Tensor:
+    """The E2M3 pattern whose value is q + 1/2, for INT4 codes q in [-8, 7] (found by search over all 64 patterns)."""
+    table = e2m3_value(torch.arange(64))
+    want = q.to(torch.float64) + .5
+    hit = table[None, :] == want.reshape(-1, 1)
+    assert bool(hit.any(dim=1).all()), 'a code whose q + 1/2 is not an E2M3 value'
+    return hit.to(torch.int64).argmax(dim=1).reshape(q.shape).to(torch.uint8)
+
+
+def _tile_index(rows: int, k: int):
+    """For every (row, k) of a code matrix: byte-independent coordinates (fragment, lane, position in the lane's 32)."""
+    r = torch.arange(rows)[:, None].expand(rows, k)
+    c = torch.arange(k)[None, :].expand(rows, k)
+    frag = (r // 32) * (k // 64) + c // 64
+    lane = 32 * ((c % 64) // 32) + r % 32
+    return frag, lane, c % 32
+
+
+def e2m3_tiles_encode(x_int: torch.Tensor) -> torch.Tensor:
+    """(rows, K) int8 codes -> flat uint8 E2M3 tiles (layout of include/quest_hip.h; padding rows are zero bytes)."""
+    rows, k = x_int.shape
+    assert k % 64 == 0
+    nfrag = ((rows + 31) // 32) * (k // 64)
+    frag, lane, j = _tile_index(rows, k)
+    bits = e2m3_bits_of_code(x_int).to(torch.int64)
+    # the lane's 24 bytes as a bit string: code j at bits [6 j, 6 j + 6); spread into (nfrag, 64, 192) single bits
+    lane_bits = torch.zeros(nfrag, 64, 192, dtype=torch.uint8)
+    for b in range(6):
+        lane_bits[frag, lane, 6 * j + b] = ((bits >> b) & 1).to(torch.uint8)
+    weights = (1 << torch.arange(8)).to(torch.uint8)
+    lane_bytes = (lane_bits.view(nfrag, 64, 24, 8) * weights).sum(dim=-1).to(torch.uint8)     # (nfrag, 64, 24)
+    out = torch.empty(nfrag, E2M3_FRAGMENT_BYTES, dtype=torch.uint8)
+    out[:, :1024] = lane_bytes[:, :, :16].reshape(nfrag, 1024)
+    out[:, 1024:] = lane_bytes[:, :, 16:].reshape(nfrag, 512)
+    return out.reshape(-1)
+
+
+def e2m3_tiles_decode(tiles: torch.Tensor, rows: int, k: int) -> torch.Tensor:
+    """Flat uint8 E2M3 tiles -> (rows, K) fp64 values (q + 1/2 for tiles that hold codes)."""
+    nfrag = ((rows + 31) // 32) * (k // 64)
+    t = tiles.reshape(nfrag, E2M3_FRAGMENT_BYTES)
+    lane_bytes = torch.cat((t[:, :1024].reshape(nfrag, 64, 16), t[:, 1024:].reshape(nfrag, 64, 8)), dim=2)
+    lane_bits = ((lane_bytes[..., None].to(torch.int64) >> torch.arange(8)) & 1).reshape(nfrag, 64, 192)
+    frag, lane, j = _tile_index(rows, k)
+    bits = torch.zeros(rows, k, dtype=torch.int64)
+    for b in range(6):
+        bits |= lane_bits[frag, lane, 6 * j + b] << b
+    return e2m3_value(bits)
+
+
+# ---------------------------------------------------------------------------------------------
 # The training-side (fake-quantised) statement of the same layer, for judging the packed INT4 path
 # against what a QuEST-trained checkpoint was evaluated with.
 # ---------------------------------------------------------------------------------------------

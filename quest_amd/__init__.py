@@ -24,6 +24,9 @@ from .api import (  # noqa: F401
     rope_interleaved_,
     silu_mul_hadamard_quantize_int4,
     uncompress_meta48_int4,
+    e2m3_tiles_bytes,
+    int4_to_e2m3_tiles,
+    fused_matmul_dequantize_e2m3,
 )
 
 __version__ = '0.1.0'

@@ -19,7 +19,7 @@ DTYPE_CODE = {torch.bfloat16: QUEST_DTYPE_BF16, torch.float16: QUEST_DTYPE_FP16}
 
 _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
-# name -> argtypes; every function returns int except quest_status_string
+# name -> argtypes; every function returns an int status unless _RESTYPES says otherwise
 SIGNATURES = {
     'quest_version': [],
     'quest_status_string': [_i],
@@ -36,7 +36,13 @@ SIGNATURES = {
     'quest_hadamard_quantize_int4_rule': [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
     'quest_rope_interleaved': [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     'quest_silu_mul_hadamard_quantize_int4': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
+    'quest_e2m3_tiles_bytes': [_i, _i],
+    'quest_int4_to_e2m3_tiles': [_vp, _vp, _i, _i, _vp],
+    'quest_fused_matmul_dequantize_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    'quest_fused_matmul_dequantize_swiglu_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
 }
+# entry points that do not return an int status
+_RESTYPES = {'quest_status_string': ctypes.c_char_p, 'quest_e2m3_tiles_bytes': ctypes.c_size_t}
 
 _lib = None
 
@@ -53,7 +59,7 @@ def load() -> ctypes.CDLL:
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
-            fn.restype = ctypes.c_char_p if name == 'quest_status_string' else ctypes.c_int
+            fn.restype = _RESTYPES.get(name, ctypes.c_int)
         _lib = lib
     return _lib
 

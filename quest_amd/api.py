@@ -341,3 +341,55 @@ def rope_interleaved_(x: torch.Tensor, freqs_cis: torch.Tensor, rot_cols: int, h
         check(_lib.load().quest_rope_interleaved(ptr(x), ptr(freqs_cis), b * t, t, c, rot_cols, head_dim,
                                                  DTYPE_CODE[x.dtype], stream_of(x)), 'rope_interleaved')
     return x
+
+
+# ---- the FP6 matrix-core path: codes kept as "E2M3 tiles" (see include/quest_hip.h) ---------------------------------
+def e2m3_tiles_bytes(rows: int, k: int) -> int:
+    """Bytes of the E2M3 tiles of a (rows, k) code matrix."""
+    n = _lib.load().quest_e2m3_tiles_bytes(rows, k)
+    if n == 0:
+        raise RuntimeError(f'E2M3 tiles need rows > 0 and K % 64 == 0; got ({rows}, {k})')
+    return n
+
+
+def int4_to_e2m3_tiles(x_int_packed: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """Packed INT4 codes (rows, K/2) uint8 -> their E2M3 tiles (flat uint8): the operand form of
+    `fused_matmul_dequantize_e2m3`, each code q stored as the FP6 E2M3 value q + 1/2."""
+    rows, k = x_int_packed.size(0), x_int_packed.size(1) * 2
+    if out is None:
+        out = torch.empty(e2m3_tiles_bytes(rows, k), dtype=torch.uint8, device=x_int_packed.device)
+    assert x_int_packed.dtype == torch.uint8 and x_int_packed.is_contiguous() and x_int_packed.dim() == 2
+    assert out.dtype == torch.uint8 and out.is_contiguous() and out.numel() == e2m3_tiles_bytes(rows, k)
+    dev = require_gpu(x_int_packed, out)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_int4_to_e2m3_tiles(ptr(out), ptr(x_int_packed), rows, k, stream_of(out)), 'int4_to_e2m3_tiles')
+    return out
+
+
+def fused_matmul_dequantize_e2m3(
+        a_tiles: torch.Tensor,
+        b_tiles: torch.Tensor,
+        vec_a_mul: torch.Tensor,
+        vec_b_mul: torch.Tensor,
+        size_k: int,
+        out: torch.Tensor = None,
+        swiglu: bool = False,
+) -> torch.Tensor:
+    """`fused_matmul_dequantize_int4_int4t_bf16` for codes held as E2M3 tiles: (M, N) outputs identical bit for bit,
+    from the FP6 matrix instructions; the add vectors are not needed (2 C + a_add + b_add is twice the FP6 sum).
+    M and N are the lengths of the scale vectors.  swiglu=True: the epilogue of
+    `fused_matmul_dequantize_swiglu_int4_int4t`, b in its interleaved row order, (M, N / 2) outputs."""
+    m, n = vec_a_mul.numel(), vec_b_mul.numel()
+    if out is None:
+        out = torch.empty(m, n // 2 if swiglu else n, dtype=vec_a_mul.dtype, device=a_tiles.device)
+    assert a_tiles.dtype == torch.uint8 and b_tiles.dtype == torch.uint8 and a_tiles.is_contiguous() and b_tiles.is_contiguous()
+    assert a_tiles.numel() == e2m3_tiles_bytes(m, size_k) and b_tiles.numel() == e2m3_tiles_bytes(n, size_k)
+    assert vec_a_mul.dtype in _FLOAT16S and vec_b_mul.dtype == vec_a_mul.dtype and out.dtype == vec_a_mul.dtype
+    assert vec_a_mul.is_contiguous() and vec_b_mul.is_contiguous() and out.is_contiguous()
+    assert out.shape == (m, n // 2 if swiglu else n)
+    dev = require_gpu(a_tiles, b_tiles, vec_a_mul, vec_b_mul, out)
+    fn = _lib.load().quest_fused_matmul_dequantize_swiglu_e2m3 if swiglu else _lib.load().quest_fused_matmul_dequantize_e2m3
+    with torch.cuda.device(dev):
+        check(fn(ptr(out), ptr(a_tiles), ptr(b_tiles), ptr(vec_a_mul), ptr(vec_b_mul), m, size_k, n,
+                 DTYPE_CODE[out.dtype], stream_of(out)), 'fused_matmul_dequantize_e2m3')
+    return out

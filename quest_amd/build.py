@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 LIB_PATH = os.path.join(HERE, 'libquest_hip.so')
 SOURCES = ['rowops.hip', 'hadamard_mfma.hip', 'gemm.hip', 'gemm_big.hip', 'gemm_small.hip', 'gemm_staged.hip',
-           'gemm_decode.hip', 'capi.hip']
+           'gemm_decode.hip', 'gemm_e2m3.hip', 'capi.hip']
 
 FLAGS = [
     '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-shared',

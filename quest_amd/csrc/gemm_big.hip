@@ -12,18 +12,9 @@
 // and splits them into the int8 vectors of 16 * (even-k nibbles) and 16 * (odd-k nibbles), which
 // feed two MFMA k-steps.  The stage pipeline runs on across the workgroup's tiles, and the
 // epilogue's stores are left to drain under the next tile's first stages.
-#include "gemm_tiles.h"
+#include "gemm_schedule.h"
 
 namespace quest {
-
-// How a persistent grid divides the (token tile, channel unit) cells among its workgroups.
-struct Schedule {
-    int tiles_t;        // token tiles of 256
-    int units;          // channel units of 32
-    int groups;         // channel super-groups (one per XCD when the grid allows)
-    int row_tiles;      // > 0: one tile per workgroup, this many per token tile of a group (0: contiguous runs of cells)
-    int by_tokens;      // the groups divide the token tiles among them (and each takes all channel units) instead of the units
-};
 
 namespace big {
 
@@ -53,34 +44,6 @@ struct Cfg {
 };
 using Wide = Cfg<8, 4, 1>;
 using Duo = Cfg<4, 3, 2>;
-
-struct Cursor {          // walks a workgroup's run of cells tile by tile, stage by stage (no divisions)
-    int tt, u;               // next cell: token tile, channel unit inside the group
-    int left;                // cells left in the run
-    int nug, ug0;
-    int tok0, ch0, width;    // current tile
-    int kt;                  // next stage of the current tile
-    bool valid;
-};
-
-template <typename C>
-__device__ __forceinline__ void cursor_next_tile(Cursor &c) {
-    if (c.left <= 0) { c.valid = false; return; }             // keeps pointing at the last tile
-    int width = c.nug - c.u;
-    width = width < c.left ? width : c.left;
-    // kept in a scalar register: two chained minima would otherwise be selected as the vector ALU's three-operand
-    // minimum, which drags the whole cursor into vector registers (and those get spilled at the register peaks)
-    asm volatile("" : "+s"(width));
-    width = width < C::kMaxUnits ? width : C::kMaxUnits;
-    c.tok0 = c.tt * kRows;
-    c.ch0 = (c.ug0 + c.u) * 32;
-    c.width = width;
-    c.kt = 0;
-    c.valid = true;
-    c.left -= width;
-    c.u += width;
-    if (c.u == c.nug) { c.u = 0; c.tt++; }
-}
 
 struct Loader {          // direct-to-LDS loads of one wave: 4 instructions of 16 token rows, 2 or 4 of 16 channel rows
     __amdgpu_buffer_rsrc_t act, wgt, badd, bmul, aadd, amul;
@@ -121,7 +84,7 @@ template <typename C>
 __device__ __forceinline__ void loader_end(Loader &l, Cursor &ld) {
     l.issued++;
     if (++ld.kt == l.nk) {
-        cursor_next_tile<C>(ld);
+        cursor_next_tile<C::kMaxUnits>(ld);
         if (ld.valid) loader_offsets<C>(l, ld, fresh_lane_id()); else ld.kt = l.nk - 1;
     }
 }
@@ -512,51 +475,12 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
     const int wc = wave & 1;                     // channel half this wave multiplies
     const int kbytes = K >> 1;
 
-    const int rank = __builtin_amdgcn_readfirstlane((int)(blockIdx.x / sch.groups));
-    const int grp = blockIdx.x - rank * sch.groups;
-    const int per_grp = __builtin_amdgcn_readfirstlane((int)(gridDim.x / sch.groups));
-    // A group (= an XCD and its L2 when there are eight) owns a slice of the channel units and all token tiles, or --
-    // by_tokens -- a slice of the token tiles and all units: whichever operand is the smaller one is then the one every
-    // XCD fetches whole (and keeps in its L2), and the larger one is fetched once in total.
-    int ug0 = 0, ug1 = sch.units, tt_lo = 0, tt_hi = sch.tiles_t;
-    if (sch.by_tokens) {
-        tt_lo = __builtin_amdgcn_readfirstlane((int)(((long)grp * sch.tiles_t) / sch.groups));
-        tt_hi = __builtin_amdgcn_readfirstlane((int)(((long)(grp + 1) * sch.tiles_t) / sch.groups));
-    } else {
-        ug0 = __builtin_amdgcn_readfirstlane((int)(((long)grp * sch.units) / sch.groups));
-        ug1 = __builtin_amdgcn_readfirstlane((int)(((long)(grp + 1) * sch.units) / sch.groups));
-    }
     Cursor cc, ld;
-    cc.nug = ug1 - ug0;
-    cc.ug0 = ug0;
-    // the divisions run on the vector ALU (there is no scalar divide); readfirstlane brings the (uniform) results
-    // back to scalar registers, and with them the whole cursor arithmetic of the tile loop
-    const long cells = (long)(tt_hi - tt_lo) * cc.nug;
-    int pos0, pos1;
-    if (sch.row_tiles > 0) {
-        // about one tile per workgroup: every token tile's units are cut into row_tiles tiles of equal width (+-1) and
-        // workgroup `rank` takes one of them.  An even split of the cells would let runs cross token-tile boundaries,
-        // and a workgroup with two tiles (each a full K loop) then takes twice as long as the others.
-        const int q = sch.row_tiles;
-        const int tile_t = __builtin_amdgcn_readfirstlane(rank / q);
-        const int i = rank - tile_t * q;
-        pos0 = tile_t * cc.nug + __builtin_amdgcn_readfirstlane((i * cc.nug) / q);
-        pos1 = tile_t * cc.nug + __builtin_amdgcn_readfirstlane(((i + 1) * cc.nug) / q);
-        if (tile_t >= sch.tiles_t) pos1 = pos0;
-    } else {
-        pos0 = __builtin_amdgcn_readfirstlane((int)((cells * rank) / per_grp));
-        pos1 = __builtin_amdgcn_readfirstlane((int)((cells * (rank + 1)) / per_grp));
-    }
-    const int tt_rel = __builtin_amdgcn_readfirstlane(pos0 / cc.nug);
-    cc.tt = tt_lo + tt_rel;
-    cc.u = pos0 - tt_rel * cc.nug;
-    cc.left = pos1 - pos0;
-    cc.valid = false;
-    cc.tok0 = cc.ch0 = cc.width = cc.kt = 0;
+    cursor_begin(sch, cc);
     ld = cc;
-    cursor_next_tile<C>(cc);
+    cursor_next_tile<C::kMaxUnits>(cc);
     if (!cc.valid) return;                       // uniform: the whole workgroup has nothing to do
-    cursor_next_tile<C>(ld);
+    cursor_next_tile<C::kMaxUnits>(ld);
 
     Loader ldr;
     ldr.act = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, M * kbytes, 0x00020000);
@@ -615,7 +539,7 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
             }
         }
 #undef QUEST_BIG_TILE
-        cursor_next_tile<C>(cc);
+        cursor_next_tile<C::kMaxUnits>(cc);
     }
     wait_vmcnt_imm<0>();                         // no direct-to-LDS load may outlive the workgroup's LDS allocation
 }
@@ -625,37 +549,8 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
 template <typename C, int OUT, bool GLU>
 static int launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                            const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
-    Schedule sch;
-    sch.tiles_t = (M + big::kRows - 1) / big::kRows;
-    sch.units = (N + 31) / 32;
-    const long cells = (long)sch.tiles_t * sch.units;
-    long grid = (long)C::kWgPerCu * cus;                      // persistent: one or two workgroups per CU
-    if (grid > cells) grid = cells;
-    sch.groups = (grid % 8 == 0 && sch.units >= 8) ? 8 : 1;
-    sch.row_tiles = 0;
-    sch.by_tokens = 0;
-    // More tokens than channels: the eight XCD groups divide the token tiles instead of the channel units, so that the
-    // weights (the smaller operand) are what every XCD fetches whole and the activation codes cross the fabric once
-    // (measured +4..7 % at M = 16384 with N = 1024..5632; no difference at M = 4096, N = 11008 either way).
-    if (M > N && grid % 8 == 0 && sch.tiles_t >= 8) {
-        sch.groups = 8;
-        sch.by_tokens = 1;
-    }
-    if (!sch.by_tokens) {
-        // few cells per workgroup: one tile each, cut along the channel units of single token tiles (see the kernel)
-        const long per_grp = grid / sch.groups;
-        const int nug = (sch.units + sch.groups - 1) / sch.groups;
-        if ((long)sch.tiles_t * nug <= (long)C::kMaxUnits * per_grp) {
-            for (int w = 1; w <= C::kMaxUnits; w++) {
-                const int q = (nug + w - 1) / w;
-                if ((long)sch.tiles_t * q <= per_grp) {
-                    sch.row_tiles = q;
-                    grid = (long)sch.groups * sch.tiles_t * q;
-                    break;
-                }
-            }
-        }
-    }
+    long grid = 0;
+    const Schedule sch = make_schedule(M, N, C::kMaxUnits, C::kWgPerCu, cus, &grid);
     big::gemm_w4a4_big_kernel<C, OUT, GLU><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
         out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
     return launch_status();

@@ -1,0 +1,174 @@
+"""GPU parity of the FP6 (E2M3) matrix-core path: the operand form of the codes and the GEMM on it, through the C ABI.
+
+Bars: the E2M3 tiles are a re-encoding of the INT4 codes (bit-exact against the oracle's encoder, and decoding them
+gives q + 1/2 for exactly the codes that went in); the GEMM's outputs equal the oracle's fused GEMM + scale epilogue
+(benchmarks/utils.py:544 on the exact integer matrix) bit for bit -- i.e. the FP6 sums are exact -- and those of the
+INT8 kernels on the same codes."""
+import pytest
+import torch
+
+from oracle import quest_oracle as qo
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16]
+DEV = 'cuda:0'
+
+
+@pytest.fixture(scope='module')
+def quest():
+    import quest_amd
+    from quest_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available()
+    return quest_amd
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16).to(torch.int32)
+
+
+def rand_codes(rows, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(-8, 8, (rows, k), generator=g).to(torch.int8)
+
+
+def scales(m, n, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return ((torch.rand(m, 1, generator=g) * 0.09 + 0.01).to(dtype), (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype))
+
+
+def oracle_output(qa, qb, a_mul, b_mul):
+    """The reference's fused GEMM on packed codes with its add vectors (the oracle's statement of utils.py:544)."""
+    k = qa.size(1)
+    a_add = qa.to(torch.int32).sum(-1, keepdim=True).to(torch.int32)
+    b_add = qb.to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2
+    return qo.fused_matmul_dequantize_int4_int4t(qo.pack_int4(qa), qo.pack_int4(qb), a_add, b_add, a_mul, b_mul, via='fp32')
+
+
+@pytest.mark.parametrize('shape', [(32, 64), (70, 128), (1, 4096), (257, 384), (4096, 1024), (33, 11008)])
+def test_tiles_are_the_oracle_encoding(quest, shape):
+    rows, k = shape
+    q = rand_codes(rows, k, 11)
+    tiles = quest.int4_to_e2m3_tiles(qo.pack_int4(q).to(DEV)).cpu()
+    assert tiles.numel() == quest.e2m3_tiles_bytes(rows, k) == ((rows + 31) // 32) * (k // 64) * 1536
+    assert torch.equal(tiles, qo.e2m3_tiles_encode(q))
+    assert torch.equal(qo.e2m3_tiles_decode(tiles, rows, k), q.double() + .5)
+
+
+GEMM_SHAPES = [(256, 128, 256), (160, 768, 224), (512, 1024, 1024), (257, 128, 300), (300, 256, 257), (33, 128, 7),
+               (1, 4096, 64), (1001, 128, 96), (777, 1152, 4100), (4097, 128, 1031), (1536, 256, 4096),
+               (4096, 256, 2048), (2048, 4096, 512), (16390, 256, 1000), (640, 2816, 1024)]
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', GEMM_SHAPES)
+def test_gemm_bit_exact(quest, dtype, shape):
+    m, k, n = shape
+    qa, qb = rand_codes(m, k, 7), rand_codes(n, k, 8)
+    a_mul, b_mul = scales(m, n, dtype, 6)
+    want = oracle_output(qa, qb, a_mul, b_mul)
+    ta = quest.int4_to_e2m3_tiles(qo.pack_int4(qa).to(DEV))
+    tb = quest.int4_to_e2m3_tiles(qo.pack_int4(qb).to(DEV))
+    got = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul.to(DEV), b_mul.to(DEV), k).cpu()
+    assert got.dtype == dtype and got.shape == (m, n)
+    assert torch.equal(bits(got), bits(want))
+    ref = qo.linear_fp64(qa, a_mul, qb, b_mul)
+    assert ((got.double() - ref).norm() / ref.norm()) < 1e-2
+
+
+def test_every_pair_of_codes(quest):
+    """Row i of A holds code (i % 16) in every position, row j of B code (j % 16): all 256 products, each summed K times."""
+    k = 256
+    qa = (torch.arange(32) % 16 - 8).to(torch.int8)[:, None].repeat(1, k)
+    qb = (torch.arange(48) % 16 - 8).to(torch.int8)[:, None].repeat(1, k)
+    one = torch.ones(32, 1, dtype=torch.float16), torch.ones(48, 1, dtype=torch.float16)
+    ta = quest.int4_to_e2m3_tiles(qo.pack_int4(qa).to(DEV))
+    tb = quest.int4_to_e2m3_tiles(qo.pack_int4(qb).to(DEV))
+    got = quest.fused_matmul_dequantize_e2m3(ta, tb, one[0].to(DEV), one[1].to(DEV), k).cpu().double()
+    want = k * (qa[:, :1].double() + .5) @ (qb[:, :1].double() + .5).t()        # |.| <= 256 * 56.25: exact in fp16
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize('k', [11008, 65536])
+def test_extreme_sums_are_exact(quest, k):
+    """All codes -8 against -8 and against 7: the largest sums the path can see (56.25 K), then half a row of large
+    products followed by small random ones (a large accumulator must not swallow the quarter units)."""
+    m, n = 64, 96
+    qa = torch.full((m, k), -8, dtype=torch.int8)
+    qb = torch.full((n, k), -8, dtype=torch.int8)
+    qb[1::2] = 7
+    qa[32:, k // 2:] = rand_codes(32, k // 2, 3)
+    qb[48:, k // 2:] = rand_codes(48, k // 2, 4)
+    a_mul, b_mul = scales(m, n, torch.bfloat16, 9)
+    ta = quest.int4_to_e2m3_tiles(qo.pack_int4(qa).to(DEV))
+    tb = quest.int4_to_e2m3_tiles(qo.pack_int4(qb).to(DEV))
+    got = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul.to(DEV), b_mul.to(DEV), k).cpu()
+    assert torch.equal(bits(got), bits(oracle_output(qa, qb, a_mul, b_mul)))
+
+
+@pytest.mark.parametrize('seed', range(12))
+def test_gemm_seeded_fuzz(quest, seed):
+    g = torch.Generator().manual_seed(1000 + seed)
+    m = int(torch.randint(1, 1200, (1,), generator=g))
+    n = int(torch.randint(1, 1500, (1,), generator=g))
+    k = 128 * int(torch.randint(1, 24, (1,), generator=g))
+    dtype = DTYPES[seed % 2]
+    qa, qb = rand_codes(m, k, 2000 + seed), rand_codes(n, k, 3000 + seed)
+    a_mul, b_mul = scales(m, n, dtype, 4000 + seed)
+    ta = quest.int4_to_e2m3_tiles(qo.pack_int4(qa).to(DEV))
+    tb = quest.int4_to_e2m3_tiles(qo.pack_int4(qb).to(DEV))
+    got = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul.to(DEV), b_mul.to(DEV), k).cpu()
+    assert torch.equal(bits(got), bits(oracle_output(qa, qb, a_mul, b_mul))), (m, k, n)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_gemm_equals_int8_kernels_at_prefill_size(quest, dtype):
+    """M = 4096, K = 4096, N = 11008: the whole output against the INT8 kernel on the same codes (itself checked against
+    exact integers at this size), bit for bit."""
+    m, k, n = 4096, 4096, 11008
+    g = torch.Generator(device=DEV).manual_seed(5)
+    a = torch.randint(0, 256, (m, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    b = torch.randint(0, 256, (n, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    a_mul = (torch.rand(m, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    from quest_amd import harness
+    a_add = harness.unpack_int4(a).to(torch.int32).sum(-1, keepdim=True).to(torch.int32)
+    b_add = harness.unpack_int4(b).to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2
+    want = quest.fused_matmul_dequantize_int4_int4t_bf16(a, b, a_add, b_add, a_mul, b_mul)
+    got = quest.fused_matmul_dequantize_e2m3(quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(b), a_mul, b_mul, k)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    again = quest.fused_matmul_dequantize_e2m3(quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(b), a_mul, b_mul, k)
+    assert torch.equal(got.view(torch.int16), again.view(torch.int16))
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(160, 768, 224), (300, 256, 1000), (4096, 128, 4104), (1000, 512, 2048)])
+def test_gemm_swiglu_equals_int8_kernel(quest, dtype, shape):
+    m, k, n = shape
+    h = n // 2
+    qa, qb = rand_codes(m, k, 31), rand_codes(n, k, 32)
+    a_mul, b_mul = scales(m, n, dtype, 33)
+    a, b = qo.pack_int4(qa).to(DEV), qo.pack_int4(qb).to(DEV)
+    a_add = qa.to(torch.int32).sum(-1, keepdim=True).to(torch.int32).to(DEV)
+    b_add = (qb.to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2).to(DEV)
+    p = quest.swiglu_interleave_rows(h, device=DEV)
+    bp, bp_add, bp_mul = b[p].contiguous(), b_add[p].contiguous(), b_mul.to(DEV)[p].contiguous()
+    want = quest.fused_matmul_dequantize_swiglu_int4_int4t(a, bp, a_add, bp_add, a_mul.to(DEV), bp_mul)
+    got = quest.fused_matmul_dequantize_e2m3(quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(bp), a_mul.to(DEV), bp_mul, k,
+                                             swiglu=True)
+    assert got.shape == (m, h)
+    assert torch.equal(bits(got.cpu()), bits(want.cpu()))
+
+
+def test_error_codes(quest):
+    from quest_amd import _lib
+    import ctypes
+    lib = _lib.load()
+    null, fake = ctypes.c_void_p(0), ctypes.c_void_p(0x1000)
+    assert lib.quest_fused_matmul_dequantize_e2m3(fake, fake, fake, fake, null, 4, 128, 4, 0, null) == -1
+    assert lib.quest_fused_matmul_dequantize_e2m3(fake, fake, fake, fake, fake, 4, 192, 4, 0, null) == -2
+    assert lib.quest_fused_matmul_dequantize_e2m3(fake, fake, fake, fake, fake, 4, 1 << 17, 4, 0, null) == -5
+    assert lib.quest_fused_matmul_dequantize_e2m3(fake, fake, fake, fake, fake, 4, 128, 4, 7, null) == -3
+    assert lib.quest_int4_to_e2m3_tiles(fake, fake, 4, 100, null) == -2
+    assert lib.quest_e2m3_tiles_bytes(4, 100) == 0
