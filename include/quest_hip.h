@@ -151,7 +151,7 @@ int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *
  * attention and MLP block of the reference's model (src/models/llama.py:71-77, applied at llama.py:174-175) --
  * then Hadamard, scale, codes, row sums of y as above.  x_norm, when not NULL, receives y.  No counterpart in
  * the reference's quest package, which quantises a tensor the norm has already written.
- * group_size % 128 == 0, group_size <= 4096, had_scale exactly representable in dtype (181/2048 is);
+ * group_size % 128 == 0, group_size <= 32768, had_scale exactly representable in dtype (181/2048 is);
  * QUEST_ERR_UNSUPPORTED otherwise (the caller then runs the norm itself and quest_hadamard_quantize_int4).
  */
 int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *norm_weight, float eps, void *scale,
@@ -206,7 +206,8 @@ int quest_rope_interleaved(void *x, const float *freqs_cis, int n_rows, int seq_
  * E2M3 tiles of a (rows, size_k) code matrix, size_k % 64 == 0: ceil(rows / 32) row blocks x size_k / 64 fragments
  * of 1536 bytes, row block major.  In fragment (rb, ks), lane l = 32 g + i (row 32 rb + i, codes k = 64 ks + 32 g ..
  * + 31) owns 32 x 6 bits, code j (the E2M3 bits of q + 1/2) at bits [6 j, 6 j + 6) of its 24 bytes: bytes 0 .. 15 at
- * fragment offset 16 l, bytes 16 .. 23 at offset 1024 + 8 l.  Rows past `rows` in the last row block hold zeros.
+ * fragment offset 16 l, bytes 16 .. 23 at offset 1024 + 8 l.  Rows past `rows` in the last row block are padding: any
+ * content is valid there (E2M3 has no Inf or NaN) and no result depends on it.
  */
 
 /* Bytes of the E2M3 tiles of a (rows, size_k) code matrix; 0 for an invalid shape. */
@@ -229,6 +230,29 @@ int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_tiles, const v
 int quest_fused_matmul_dequantize_swiglu_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles,
                                               const void *vec_a_mul, const void *vec_b_mul, int size_m, int size_k,
                                               int size_n, int dtype, void *stream);
+
+/*
+ * quest_hadamard_quantize_int4 writing the codes as E2M3 tiles (x_tiles, quest_e2m3_tiles_bytes(batch_size,
+ * group_size) bytes; rows past batch_size in the last row block are left unwritten: the GEMM never uses what it
+ * computes from them).  The tiles hold exactly the codes the packed output would: x_int_packed and x_int_row_sum may
+ * be asked for as well.  Only the matrix-core form of the transform writes tiles: had_scale must be exactly
+ * representable in dtype (181/2048 is) and group_size <= 32768, QUEST_ERR_UNSUPPORTED otherwise (the caller then
+ * quantises to packed codes and converts them with quest_int4_to_e2m3_tiles).
+ */
+int quest_hadamard_quantize_e2m3(const void *x, void *scale, void *x_tiles, uint8_t *x_int_packed,
+                                 int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size, float had_scale,
+                                 int dtype, void *stream);
+
+/* quest_rmsnorm_hadamard_quantize_int4, quest_add_rmsnorm_hadamard_quantize_int4 and
+ * quest_silu_mul_hadamard_quantize_int4 with the codes written as E2M3 tiles instead of packed nibbles and row sums. */
+int quest_rmsnorm_hadamard_quantize_e2m3(const void *x, const void *norm_weight, float eps, void *scale, void *x_tiles,
+                                         void *x_norm, int group_size, int batch_size, float had_scale, int dtype,
+                                         void *stream);
+int quest_add_rmsnorm_hadamard_quantize_e2m3(void *x, const void *branch, const void *norm_weight, float eps,
+                                             void *scale, void *x_tiles, int group_size, int batch_size,
+                                             float had_scale, int dtype, void *stream);
+int quest_silu_mul_hadamard_quantize_e2m3(const void *gate_up, void *scale, void *x_tiles, void *x_act, int group_size,
+                                          int batch_size, float had_scale, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

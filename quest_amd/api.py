@@ -393,3 +393,98 @@ def fused_matmul_dequantize_e2m3(
         check(fn(ptr(out), ptr(a_tiles), ptr(b_tiles), ptr(vec_a_mul), ptr(vec_b_mul), m, size_k, n,
                  DTYPE_CODE[out.dtype], stream_of(out)), 'fused_matmul_dequantize_e2m3')
     return out
+
+
+QUEST_ERR_UNSUPPORTED = -5
+
+
+def hadamard_quantize_e2m3(
+        x: torch.Tensor,
+        scale: torch.Tensor = None,
+        x_tiles: torch.Tensor = None,
+        x_int_packed: torch.Tensor = None,
+        x_int_row_sum: torch.Tensor = None,
+        x_had: torch.Tensor = None,
+        hadamard_scale: float = HADAMARD_ENTRY,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """`hadamard_quantize_int4` with the codes written as E2M3 tiles (one pass over x).  x_int_packed / x_int_row_sum,
+    if given, receive the packed form of the same codes as well.  Shapes the matrix-core kernel does not take (no
+    transform, the weight-side factor, rows over 32768) are quantised to packed codes first and converted.
+    Returns (scale, x_tiles)."""
+    m, k = x.shape
+    if scale is None:
+        scale = torch.empty(m, 1, dtype=x.dtype, device=x.device)
+    if x_tiles is None:
+        x_tiles = torch.empty(e2m3_tiles_bytes(m, k), dtype=torch.uint8, device=x.device)
+    assert x.dtype in _FLOAT16S and x.is_contiguous() and scale.dtype == x.dtype and scale.is_contiguous() and scale.numel() == m
+    assert x_tiles.dtype == torch.uint8 and x_tiles.is_contiguous() and x_tiles.numel() == e2m3_tiles_bytes(m, k)
+    assert x_int_packed is None or (x_int_packed.dtype == torch.uint8 and x_int_packed.is_contiguous() and x_int_packed.shape == (m, k // 2))
+    assert x_int_row_sum is None or (x_int_row_sum.dtype == torch.int32 and x_int_row_sum.is_contiguous() and x_int_row_sum.numel() == m)
+    assert x_had is None or (x_had.dtype == x.dtype and x_had.shape == x.shape and x_had.is_contiguous())
+    dev = require_gpu(x, scale, x_tiles, x_int_packed, x_int_row_sum, x_had)
+    with torch.cuda.device(dev):
+        rc = _lib.load().quest_hadamard_quantize_e2m3(ptr(x), ptr(scale), ptr(x_tiles), ptr(x_int_packed), ptr(x_int_row_sum),
+                                                      ptr(x_had), k, m, float(hadamard_scale), DTYPE_CODE[x.dtype], stream_of(x))
+    if rc == QUEST_ERR_UNSUPPORTED:
+        _, packed, _ = hadamard_quantize_int4(x, scale, x_int_packed, x_int_row_sum, x_had, hadamard_scale=hadamard_scale)
+        int4_to_e2m3_tiles(packed, x_tiles)
+    else:
+        check(rc, 'hadamard_quantize_e2m3')
+    return scale, x_tiles
+
+
+def _e2m3_outputs(m, k, dtype, device, scale, x_tiles):
+    if scale is None:
+        scale = torch.empty(m, 1, dtype=dtype, device=device)
+    if x_tiles is None:
+        x_tiles = torch.empty(e2m3_tiles_bytes(m, k), dtype=torch.uint8, device=device)
+    assert scale.dtype == dtype and scale.is_contiguous() and scale.numel() == m
+    assert x_tiles.dtype == torch.uint8 and x_tiles.is_contiguous() and x_tiles.numel() == e2m3_tiles_bytes(m, k)
+    return scale, x_tiles
+
+
+def rmsnorm_hadamard_quantize_e2m3(x, norm_weight, eps, scale=None, x_tiles=None, x_norm=None,
+                                   hadamard_scale: float = HADAMARD_ENTRY) -> tuple[torch.Tensor, torch.Tensor]:
+    """`rmsnorm_hadamard_quantize_int4` with the codes written as E2M3 tiles.  Returns (scale, x_tiles)."""
+    m, k = x.shape
+    assert x.dtype in _FLOAT16S and x.is_contiguous() and norm_weight.dtype == x.dtype and norm_weight.numel() == k and norm_weight.is_contiguous()
+    assert x_norm is None or (x_norm.dtype == x.dtype and x_norm.shape == x.shape and x_norm.is_contiguous())
+    scale, x_tiles = _e2m3_outputs(m, k, x.dtype, x.device, scale, x_tiles)
+    dev = require_gpu(x, norm_weight, scale, x_tiles, x_norm)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_rmsnorm_hadamard_quantize_e2m3(
+            ptr(x), ptr(norm_weight), float(eps), ptr(scale), ptr(x_tiles), ptr(x_norm), k, m, float(hadamard_scale),
+            DTYPE_CODE[x.dtype], stream_of(x)), 'rmsnorm_hadamard_quantize_e2m3')
+    return scale, x_tiles
+
+
+def add_rmsnorm_hadamard_quantize_e2m3(x, branch, norm_weight, eps, scale=None, x_tiles=None,
+                                       hadamard_scale: float = HADAMARD_ENTRY) -> tuple[torch.Tensor, torch.Tensor]:
+    """`add_rmsnorm_hadamard_quantize_int4` (x += branch in place, then the norm) with the codes written as E2M3 tiles."""
+    m, k = x.shape
+    assert x.dtype in _FLOAT16S and x.is_contiguous() and branch.dtype == x.dtype and branch.shape == x.shape
+    assert branch.is_contiguous() and branch.data_ptr() != x.data_ptr()
+    assert norm_weight.dtype == x.dtype and norm_weight.numel() == k and norm_weight.is_contiguous()
+    scale, x_tiles = _e2m3_outputs(m, k, x.dtype, x.device, scale, x_tiles)
+    dev = require_gpu(x, branch, norm_weight, scale, x_tiles)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_add_rmsnorm_hadamard_quantize_e2m3(
+            ptr(x), ptr(branch), ptr(norm_weight), float(eps), ptr(scale), ptr(x_tiles), k, m, float(hadamard_scale),
+            DTYPE_CODE[x.dtype], stream_of(x)), 'add_rmsnorm_hadamard_quantize_e2m3')
+    return scale, x_tiles
+
+
+def silu_mul_hadamard_quantize_e2m3(gate_up, scale=None, x_tiles=None, x_act=None,
+                                    hadamard_scale: float = HADAMARD_ENTRY) -> tuple[torch.Tensor, torch.Tensor]:
+    """`silu_mul_hadamard_quantize_int4` with the codes written as E2M3 tiles.  Returns (scale, x_tiles)."""
+    m, k2 = gate_up.shape
+    k = k2 // 2
+    assert gate_up.dtype in _FLOAT16S and gate_up.is_contiguous() and k2 == 2 * k
+    assert x_act is None or (x_act.dtype == gate_up.dtype and x_act.shape == (m, k) and x_act.is_contiguous())
+    scale, x_tiles = _e2m3_outputs(m, k, gate_up.dtype, gate_up.device, scale, x_tiles)
+    dev = require_gpu(gate_up, scale, x_tiles, x_act)
+    with torch.cuda.device(dev):
+        check(_lib.load().quest_silu_mul_hadamard_quantize_e2m3(
+            ptr(gate_up), ptr(scale), ptr(x_tiles), ptr(x_act), k, m, float(hadamard_scale), DTYPE_CODE[gate_up.dtype],
+            stream_of(gate_up)), 'silu_mul_hadamard_quantize_e2m3')
+    return scale, x_tiles

@@ -265,6 +265,19 @@ __device__ __forceinline__ int quant_top_nibble_any(float x, float inv28) {
     asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(tn));
     return q;
 }
+// floor of the same nudged quotient as a float, unclamped, on the low / high half of a dword of two 16-bit floats: for
+// consumers whose next conversion saturates (the FP6 operand form).  x finite and s in the fast range, as above.
+template <int DT, int HI>
+__device__ __forceinline__ float quant_floor_half(uint32_t w, float inv) {
+    float t;
+    if constexpr (DT == QUEST_DTYPE_BF16) {
+        t = __fmul_rn(HI ? hi_f32<DT>(w) : lo_f32<DT>(w), inv);
+    } else {
+        if constexpr (HI) asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(t) : "v"(w), "v"(inv));
+        else asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(w), "v"(inv));
+    }
+    return __builtin_floorf(__builtin_fmaf(__builtin_fabsf(t), 4.76837158203125e-07f, t));
+}
 // appends the nibble in the top four bits of `n` below the nibbles already in `packed` (which move up by four bits)
 __device__ __forceinline__ uint32_t push_top_nibble(uint32_t packed, int n) {
     return __builtin_amdgcn_alignbit(packed, (uint32_t)n, 28);
@@ -288,7 +301,7 @@ int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t 
 // front (pre: 0 none, 1 RMSNorm, 2 SiLU(gate) * up); QUEST_ERR_UNSUPPORTED when it does not apply
 int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
                                   int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
-                                  hipStream_t st, const void *add_in = nullptr, void *sum_out = nullptr);
+                                  hipStream_t st, const void *add_in = nullptr, void *sum_out = nullptr, uint8_t *tiles = nullptr);
 
 inline int check_dtype(int dtype) { return dtype == QUEST_DTYPE_BF16 || dtype == QUEST_DTYPE_FP16; }
 inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

@@ -15,7 +15,7 @@
 // one fragment each, row block major; a fragment is the 1536-byte register image of one MFMA operand: lane
 // l = 32 g + i (row 32 rb + i, k = 64 ks + 32 g ... + 31) owns 32 codes x 6 bits = 24 bytes, code j at bits
 // [6 j, 6 j + 6) -- its first 16 bytes at fragment byte 16 l ("head"), its last 8 at byte 1024 + 8 l ("tail").  Rows past
-// R inside the last row block hold zeros.  Global memory -> LDS is then a linear copy (direct loads, 1 KiB per wave
+// R inside the last row block are padding (any bits are finite E2M3 values and no stored result depends on them).  Global memory -> LDS is then a linear copy (direct loads, 1 KiB per wave
 // instruction) and LDS -> registers one ds_read_b128 + one ds_read_b64 per fragment at lane-linear addresses: no bank
 // conflicts, no swizzle, and nothing for the vector ALU to do in the main loop.
 //

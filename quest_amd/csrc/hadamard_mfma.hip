@@ -21,7 +21,14 @@
 // After the MFMAs lane (n, h) holds outputs 32 mt + 8 q + 4 h + e of block n: the row never leaves
 // registers.  Rows longer than 4096 are split over the waves of a workgroup, which exchange only
 // their partial sums of squares and of codes through LDS.
+//
+// Besides (or instead of) packed nibbles the codes can be written as E2M3 tiles, the operand form of the FP6 GEMM
+// (gemm_e2m3.hip; layout in include/quest_hip.h): the two half-waves trade the rounded outputs so that a lane holds
+// two whole groups of 32 consecutive k, each output becomes the fp16 value q + 1/2 (floor of the same nudged quotient
+// the nibble path converts; the clamp is the saturation of the FP6 conversion) and v_cvt_scalef32_pk32_fp6_f16 packs
+// 32 of them into the lane's 24 bytes of its fragment.
 #include "common.h"
+#include <type_traits>
 
 namespace quest {
 namespace hq {
@@ -98,8 +105,9 @@ __global__ void __launch_bounds__(64 * Shape<WPR>::kWaves, Shape<WPR>::kMinBlock
 hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ norm_w,
                               uint16_t *__restrict__ scale, uint32_t *__restrict__ packed, int32_t *__restrict__ row_sum,
                               uint16_t *__restrict__ x_had, uint16_t *__restrict__ pre_out, const uint16_t *add_in,
-                              uint16_t *sum_out, int K, int M, int ldx, uint32_t entry_bits, float eps) {
-    static_assert(WPR == 1 || (G == 32 && PRE == kPreNone), "rows shared by waves: whole waves, no producer");
+                              uint16_t *sum_out, uint8_t *__restrict__ tiles, int xcd_chunk, int K, int M, int ldx,
+                              uint32_t entry_bits, float eps) {
+    static_assert(WPR == 1 || G == 32, "rows shared by waves: whole waves");
     constexpr int kRows = Shape<WPR>::kRows;
     constexpr int kRowsPerWave = 32 / G;
     const int lane = threadIdx.x & 63;
@@ -108,7 +116,12 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
     const int row_local = wave / WPR;
     const int n = lane & 31;                   // MFMA column
     const int h = lane >> 5;
-    const int row = (blockIdx.x * kRows + row_local) * kRowsPerWave + n / G;
+    // xcd_chunk > 0 (E2M3 tiles are written): workgroups are dealt to the eight XCDs in turn, so workgroup b of the grid
+    // takes the rows of virtual workgroup (b % 8) * xcd_chunk + b / 8 -- each XCD then works through one contiguous
+    // range of rows, and the 8 (16) consecutive rows that share a 128-byte line of a fragment's heads (tails) are
+    // written through one L2 within a short time, where the partial lines merge
+    const int vb = xcd_chunk > 0 ? (int)(blockIdx.x & 7) * xcd_chunk + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const int row = (vb * kRows + row_local) * kRowsPerWave + n / G;
     const int blk = part * 32 + n % G;         // block of the row in this column
     const bool live = row < M && blk < (K >> 7);
 
@@ -181,7 +194,16 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
         for (int s = 0; s < 8; s++)
 #pragma unroll
             for (int d = 0; d < 4; d++) ss = dot2_self<DT>(bq[s][d], ss);
-        const float mean_sq = __fmul_rn(group_sum_f<G>(ss), __fdiv_rn(1.0f, (float)K));
+        float ss_row = group_sum_f<G>(ss);
+        if constexpr (WPR > 1) {                 // the row's waves add their parts in wave order: the same bits in each
+            __shared__ float part_pre[Shape<WPR>::kWaves];
+            if (lane == 0) part_pre[wave] = ss_row;
+            __syncthreads();
+            ss_row = 0.f;
+#pragma unroll
+            for (int w = 0; w < WPR; w++) ss_row += part_pre[row_local * WPR + w];
+        }
+        const float mean_sq = __fmul_rn(ss_row, __fdiv_rn(1.0f, (float)K));
         const float r = __frsqrt_rn(__fadd_rn(mean_sq, eps));
 #pragma unroll
         for (int s = 0; s < 8; s++)
@@ -261,6 +283,51 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
                 *reinterpret_cast<uint2 *>(dst + 32 * mt + 8 * q) = make_uint2(yb[mt][q * 2], yb[mt][q * 2 + 1]);
     }
     if (writer) scale[row] = (uint16_t)s16;
+
+    // ---- codes as E2M3 tiles.  Rounded outputs 32 mt + 8 q + 4 h + {0..3} sit in lane (n, h); after the exchange lane
+    // (n, h) holds all 32 outputs of the groups mt = 2 h and 2 h + 1: k-step 2 blk + h of the row, both halves.
+    if (tiles != nullptr) {
+        typedef _Float16 v32h __attribute__((ext_vector_type(32)));
+        typedef _Float16 v2hh __attribute__((ext_vector_type(2)));
+        typedef unsigned v6u __attribute__((ext_vector_type(6)));
+        typedef unsigned v16u __attribute__((ext_vector_type(16)));
+        const float sf_t = to_f32<DT>(s16);
+        const float inv = quant_inv(sf_t);
+        uint8_t *frag = tiles + ((size_t)(row >> 5) * (size_t)(K >> 6) + 2 * blk + h) * 1536;
+        auto emit = [&](auto fast_tag) {
+            constexpr bool kFast = decltype(fast_tag)::value;
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+                v16u hp;                            // dword d = 4 q + 2 h' + p: outputs 8 q + 4 h' + 2 p + {0, 1} of the group
+#pragma unroll
+                for (int j = 0; j < 8; j++) {       // j = 2 q + p
+                    const auto sw = __builtin_amdgcn_permlane32_swap(yb[g][j], yb[g + 2][j], false, false);
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++) {
+                        float f0, f1;
+                        if constexpr (kFast) {
+                            f0 = quant_floor_half<DT, 0>(sw[hh], inv);
+                            f1 = quant_floor_half<DT, 1>(sw[hh], inv);
+                        } else {
+                            f0 = quant_code_inv(lo_f32<DT>(sw[hh]), inv);
+                            f1 = quant_code_inv(hi_f32<DT>(sw[hh]), inv);
+                        }
+                        // to fp16 (round towards zero saturates at +-65504 instead of overflowing), then + 1/2
+                        const v2hh c = __builtin_bit_cast(v2hh, __builtin_amdgcn_cvt_pkrtz(f0, f1)) + v2hh{(_Float16)0.5f, (_Float16)0.5f};
+                        hp[4 * (j >> 1) + 2 * hh + (j & 1)] = __builtin_bit_cast(unsigned, c);
+                    }
+                }
+                const v6u r = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(__builtin_bit_cast(v32h, hp), 1.0f);
+                if (live) {
+                    const int slot = 32 * g + (row & 31);
+                    *reinterpret_cast<uint4 *>(frag + slot * 16) = make_uint4(r[0], r[1], r[2], r[3]);
+                    *reinterpret_cast<uint2 *>(frag + 1024 + slot * 8) = make_uint2(r[4], r[5]);
+                }
+            }
+        };
+        // degenerate rows (scale zero, Inf, NaN or outside the fast range) take the clamping form, as the nibbles do
+        if (__builtin_amdgcn_ballot_w64(row < M && !quant_fast_ok(sf_t)) == 0) emit(std::true_type{}); else emit(std::false_type{});
+    }
     if (packed == nullptr && row_sum == nullptr) return;      // uniform over the workgroup
 
     // ---- codes.  Outputs 8 Q + 4 h + {0..3} (Q = 4 mt + q) give one half-word c3 c2 c1 c0 of two's-complement nibbles.
@@ -359,6 +426,7 @@ struct Args {
     void *x_had, *pre_out;
     const void *add_in;
     void *sum_out;
+    uint8_t *tiles;
     int K, M, ldx;
     uint32_t bits;
     float eps;
@@ -368,9 +436,15 @@ struct Args {
 template <int DT, int WPR, int G, int PRE>
 static void launch_shape(const Args &a) {
     constexpr int rows = hq::Shape<WPR>::kRows * (32 / G);        // rows per workgroup
-    hq::hadamard_quantize_mfma_kernel<DT, WPR, G, PRE><<<dim3((a.M + rows - 1) / rows), dim3(64 * hq::Shape<WPR>::kWaves), 0, a.st>>>(
+    int grid = (a.M + rows - 1) / rows, xcd_chunk = 0;
+    if (a.tiles != nullptr) {                                     // see the kernel: a contiguous range of rows per XCD
+        xcd_chunk = (grid + 7) / 8;
+        grid = 8 * xcd_chunk;
+    }
+    hq::hadamard_quantize_mfma_kernel<DT, WPR, G, PRE><<<dim3(grid), dim3(64 * hq::Shape<WPR>::kWaves), 0, a.st>>>(
         (const uint16_t *)a.x, (const uint16_t *)a.norm_w, (uint16_t *)a.scale, (uint32_t *)a.packed, a.row_sum,
-        (uint16_t *)a.x_had, (uint16_t *)a.pre_out, (const uint16_t *)a.add_in, (uint16_t *)a.sum_out, a.K, a.M, a.ldx, a.bits, a.eps);
+        (uint16_t *)a.x_had, (uint16_t *)a.pre_out, (const uint16_t *)a.add_in, (uint16_t *)a.sum_out, a.tiles, xcd_chunk,
+        a.K, a.M, a.ldx, a.bits, a.eps);
 }
 
 // rows of up to 32 blocks: one wave holds 32 / G of them
@@ -387,23 +461,28 @@ static void launch_short(int g, const Args &a) {
 }
 
 // longer rows: WPR waves per row
-template <int DT>
+template <int DT, int PRE>
 static void launch_long(int wpr, const Args &a) {
     switch (wpr) {
-        case 2: launch_shape<DT, 2, 32, hq::kPreNone>(a); break;
-        case 3: launch_shape<DT, 3, 32, hq::kPreNone>(a); break;
-        case 4: launch_shape<DT, 4, 32, hq::kPreNone>(a); break;
-        case 5: launch_shape<DT, 5, 32, hq::kPreNone>(a); break;
-        case 6: launch_shape<DT, 6, 32, hq::kPreNone>(a); break;
-        case 7: launch_shape<DT, 7, 32, hq::kPreNone>(a); break;
-        default: launch_shape<DT, 8, 32, hq::kPreNone>(a); break;
+        case 2: launch_shape<DT, 2, 32, PRE>(a); break;
+        case 3: launch_shape<DT, 3, 32, PRE>(a); break;
+        case 4: launch_shape<DT, 4, 32, PRE>(a); break;
+        case 5: launch_shape<DT, 5, 32, PRE>(a); break;
+        case 6: launch_shape<DT, 6, 32, PRE>(a); break;
+        case 7: launch_shape<DT, 7, 32, PRE>(a); break;
+        default: launch_shape<DT, 8, 32, PRE>(a); break;
     }
 }
 
 template <int DT>
 static void launch_dtype(int pre, const Args &a) {
     const int nb = a.K / 128;
-    if (nb > 32) return launch_long<DT>((nb + 31) / 32, a);
+    if (nb > 32) {
+        const int wpr = (nb + 31) / 32;
+        if (pre == hq::kPreRmsNorm) return launch_long<DT, hq::kPreRmsNorm>(wpr, a);
+        if (pre == hq::kPreSiluMul) return launch_long<DT, hq::kPreSiluMul>(wpr, a);
+        return launch_long<DT, hq::kPreNone>(wpr, a);
+    }
     int g = 1;
     while (g < nb) g *= 2;
     if (pre == hq::kPreRmsNorm) launch_short<DT, hq::kPreRmsNorm>(g, a);
@@ -411,25 +490,26 @@ static void launch_dtype(int pre, const Args &a) {
     else launch_short<DT, hq::kPreNone>(g, a);
 }
 
-// Launches the matrix-core kernel when it applies (K a multiple of 128 up to 32768 -- 4096 with a producer --, a
+// Launches the matrix-core kernel when it applies (K a multiple of 128 up to 32768, a
 // Hadamard entry the dtype represents exactly); returns QUEST_ERR_UNSUPPORTED otherwise so that the caller can take
 // another path.  Whether it applies depends on K, the factor and the dtype only -- never on the number of rows or on
 // where the buffers lie -- so that one shape always runs the same arithmetic.
 // pre: 0 none, 1 RMSNorm (norm_w, eps; with add_in the norm of x + add_in, the sum written to sum_out), 2 SiLU(gate) * up
-// with x a (M, 2 K) tensor.
+// with x a (M, 2 K) tensor.  tiles: the codes as E2M3 tiles (M rows; besides or instead of packed nibbles).
 int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
                                   int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
-                                  hipStream_t st, const void *add_in, void *sum_out) {
+                                  hipStream_t st, const void *add_in, void *sum_out, uint8_t *tiles) {
     uint32_t bits = 0;
     if (K > 32768 || (K & 127) || had_scale <= 0.f || !representable16(had_scale, dtype, &bits)) return QUEST_ERR_UNSUPPORTED;
-    if (pre != hq::kPreNone && K > 4096) return QUEST_ERR_UNSUPPORTED;
     const int ldx = pre == hq::kPreSiluMul ? 2 * K : K;
     if (!aligned(pre_out, 16) || !aligned(norm_w, 16)) return QUEST_ERR_UNSUPPORTED;
     if (add_in != nullptr && (pre != hq::kPreRmsNorm || sum_out == nullptr || !aligned(add_in, 16) || !aligned(sum_out, 16)))
         return QUEST_ERR_UNSUPPORTED;
     // The kernel addresses its input with 32-bit byte offsets: tensors of 2 GiB and more go as several launches of
     // whole rows (same kernel, same arithmetic, so the result does not depend on where the cut falls).
-    const long max_rows = ((1L << 31) - 1) / ((long)ldx * 2);
+    // (cuts at multiples of 32 rows: whole row blocks of the tiles)
+    const long max_rows = (((1L << 31) - 1) / ((long)ldx * 2)) & ~31L;
+    if (max_rows == 0) return QUEST_ERR_UNSUPPORTED;
     const size_t es = 2;
     for (long r0 = 0; r0 < M; r0 += max_rows) {
         const int rows = (int)(M - r0 < max_rows ? M - r0 : max_rows);
@@ -437,7 +517,8 @@ int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, fl
             return p == nullptr ? nullptr : (void *)((const uint8_t *)p + (size_t)r0 * row_elems * elem);
         };
         const Args a = {at(x, ldx, es), norm_w, at(scale, 1, es), (uint8_t *)at(packed, K / 2, 1), (int32_t *)at(row_sum, 1, 4),
-                        at(x_had, K, es), at(pre_out, K, es), at(add_in, K, es), at(sum_out, K, es), K, rows, ldx, bits, eps, st};
+                        at(x_had, K, es), at(pre_out, K, es), at(add_in, K, es), at(sum_out, K, es),
+                        tiles == nullptr ? nullptr : tiles + (size_t)(r0 / 32) * (size_t)(K / 64) * 1536, K, rows, ldx, bits, eps, st};
         if (dtype == QUEST_DTYPE_BF16) launch_dtype<0>(pre, a);
         else launch_dtype<1>(pre, a);
     }

@@ -525,6 +525,57 @@ extern "C" int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *
                                          group_size, batch_size, had_scale, dtype, (hipStream_t)stream);
 }
 
+// ---- the same kernels writing the codes as E2M3 tiles (the operand form of gemm_e2m3.hip) -------------------------------
+static int e2m3_rows_check(const void *x, const void *scale, const void *tiles, int group_size, int batch_size, int dtype) {
+    if (!x || !scale || !tiles) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(x, 16) || !aligned(tiles, 16)) return QUEST_ERR_ALIGNMENT;
+    return QUEST_OK;
+}
+
+extern "C" int quest_hadamard_quantize_e2m3(const void *x, void *scale, void *x_tiles, uint8_t *x_int_packed,
+                                            int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size,
+                                            float had_scale, int dtype, void *stream) {
+    const int rc = e2m3_rows_check(x, scale, x_tiles, group_size, batch_size, dtype);
+    if (rc != QUEST_OK) return rc;
+    if (!aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(0, x, nullptr, 0.f, scale, x_int_packed, x_int_row_sum, x_had, nullptr, group_size,
+                                         batch_size, had_scale, dtype, (hipStream_t)stream, nullptr, nullptr, (uint8_t *)x_tiles);
+}
+
+extern "C" int quest_rmsnorm_hadamard_quantize_e2m3(const void *x, const void *norm_weight, float eps, void *scale,
+                                                    void *x_tiles, void *x_norm, int group_size, int batch_size,
+                                                    float had_scale, int dtype, void *stream) {
+    const int rc = e2m3_rows_check(x, scale, x_tiles, group_size, batch_size, dtype);
+    if (rc != QUEST_OK) return rc;
+    if (!norm_weight) return QUEST_ERR_NULL_POINTER;
+    if (!aligned(norm_weight, 16) || !aligned(x_norm, 16)) return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(1, x, norm_weight, eps, scale, nullptr, nullptr, nullptr, x_norm, group_size, batch_size,
+                                         had_scale, dtype, (hipStream_t)stream, nullptr, nullptr, (uint8_t *)x_tiles);
+}
+
+extern "C" int quest_add_rmsnorm_hadamard_quantize_e2m3(void *x, const void *branch, const void *norm_weight, float eps,
+                                                        void *scale, void *x_tiles, int group_size, int batch_size,
+                                                        float had_scale, int dtype, void *stream) {
+    const int rc = e2m3_rows_check(x, scale, x_tiles, group_size, batch_size, dtype);
+    if (rc != QUEST_OK) return rc;
+    if (!branch || !norm_weight) return QUEST_ERR_NULL_POINTER;
+    if (!aligned(branch, 16) || !aligned(norm_weight, 16)) return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(1, x, norm_weight, eps, scale, nullptr, nullptr, nullptr, nullptr, group_size, batch_size,
+                                         had_scale, dtype, (hipStream_t)stream, branch, x, (uint8_t *)x_tiles);
+}
+
+extern "C" int quest_silu_mul_hadamard_quantize_e2m3(const void *gate_up, void *scale, void *x_tiles, void *x_act,
+                                                     int group_size, int batch_size, float had_scale, int dtype,
+                                                     void *stream) {
+    const int rc = e2m3_rows_check(gate_up, scale, x_tiles, group_size, batch_size, dtype);
+    if (rc != QUEST_OK) return rc;
+    if (!aligned(x_act, 16)) return QUEST_ERR_ALIGNMENT;
+    return launch_hadamard_quantize_mfma(2, gate_up, nullptr, 0.f, scale, nullptr, nullptr, nullptr, x_act, group_size, batch_size,
+                                         had_scale, dtype, (hipStream_t)stream, nullptr, nullptr, (uint8_t *)x_tiles);
+}
+
 extern "C" int quest_rope_interleaved(void *x, const float *freqs_cis, int n_rows, int seq_len, int row_stride,
                                       int rot_cols, int head_dim, int dtype, void *stream) {
     if (!x || !freqs_cis) return QUEST_ERR_NULL_POINTER;

@@ -17,6 +17,26 @@ from .api import HADAMARD_ENTRY
 _HIP_BACKENDS = ('hip', 'triton', 'cuda')
 WEIGHT_HADAMARD_SCALE = 2. ** -3.5      # utils.py:39
 
+# Which matrix instructions the GEMM of `linear_forward` / `Linear4bit` runs on when the weight's E2M3 tiles are at
+# hand: 'fp6' = the FP6 (E2M3) kernel where it is the faster one (a few hundred tokens and more), 'int8' = always the
+# INT8 kernels on packed nibbles.  Both give the same bits.
+MATRIX_PATH = 'fp6'
+E2M3_MIN_TILES = 66                     # 256 x 256 output tiles from which the FP6 kernel is the faster one
+
+
+def prefers_e2m3(m: int, k: int, n: int) -> bool:
+    """Whether the FP6 kernel is the faster one for an (m, k) x (n, k) layer.  Its 256 x 256 tiles need about a quarter
+    of the chip's 256 compute units busy to beat the INT8 kernels' small tiles: measured over K from 1024 to 11008, N from
+    2048 to 13824 and M from 256 to 16384, the FP6 kernel wins from 66 tiles on (M = 1536 at N = 4096, M = 512 at
+    N = 11008, M = 3072 at N = 2048) and loses below 64."""
+    tiles = ((m + 255) // 256) * ((n + 255) // 256)
+    return MATRIX_PATH == 'fp6' and k % 128 == 0 and k <= 65536 and tiles >= E2M3_MIN_TILES and m * n < (1 << 31)
+
+
+def weight_tiles(w_int_packed: torch.Tensor) -> torch.Tensor:
+    """The E2M3 tiles of packed weight codes (N, K/2): the FP6 kernel's operand form (1.5 x the packed bytes)."""
+    return quest.int4_to_e2m3_tiles(w_int_packed)
+
 
 def _check_backend(backend: str) -> None:
     if backend not in _HIP_BACKENDS:
@@ -102,10 +122,12 @@ def preprocess_weight(weight: torch.Tensor, use_sparse: bool = False, use_hadama
 
 
 def linear_forward(activation, w_int_packed, w_scale, w_add, w_meta_e=None, out=None, _a_scale=None,
-                   _a_int_packed=None, _a_int_row_sum=None, _c=None, use_hadamard=False, backend='hip'):
+                   _a_int_packed=None, _a_int_row_sum=None, _c=None, use_hadamard=False, backend='hip', w_tiles=None,
+                   _a_tiles=None):
     """utils.py:56-111, dense branch: out (M, N) = quantised activation @ quantised weight^T.
     Two launches: the fused Hadamard-scale-quantise-pack kernel, then the GEMM with the scale
-    epilogue (the reference uses four)."""
+    epilogue (the reference uses four).  With `w_tiles` (`weight_tiles(w_int_packed)`) and enough tokens the codes
+    travel as E2M3 tiles and the GEMM runs on the FP6 matrix instructions: the same output bits, faster."""
     _check_backend(backend)
     if w_meta_e is not None:
         raise NotImplementedError('4:8-sparse weights are not part of this build')
@@ -113,6 +135,10 @@ def linear_forward(activation, w_int_packed, w_scale, w_add, w_meta_e=None, out=
     dtype, device = activation.dtype, activation.device
     if out is None:
         out = torch.empty(m, n, dtype=dtype, device=device)
+    if w_tiles is not None and prefers_e2m3(m, k, n):
+        a_scale, a_tiles = quest.hadamard_quantize_e2m3(activation, _a_scale, _a_tiles,
+                                                        hadamard_scale=HADAMARD_ENTRY if use_hadamard else 0.)
+        return quest.fused_matmul_dequantize_e2m3(a_tiles, w_tiles, a_scale, w_scale, k, out)
     a_scale = torch.empty(m, 1, dtype=dtype, device=device) if _a_scale is None else _a_scale
     a_int_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=device) if _a_int_packed is None else _a_int_packed
     a_int_row_sum = torch.empty(m, 1, dtype=torch.int32, device=device) if _a_int_row_sum is None else _a_int_row_sum
@@ -157,6 +183,20 @@ class Linear4bit(nn.Module):
         self.weight = torch.empty(shape, dtype=dtype, device='meta')
         for name, t in (('w_int_packed', packed), ('w_scale', scale), ('w_add', add), ('w_meta_e', None)):
             self.register_buffer(name, t)
+        self._tiles = None               # E2M3 tiles of w_int_packed: derived data, built on first use, not in checkpoints
+        self._tiles_of = None
+
+    def w_tiles(self) -> torch.Tensor:
+        """The weight codes as E2M3 tiles (built once per content of `w_int_packed`, e.g. again after a checkpoint
+        has been loaded into the buffers)."""
+        try:
+            key = (self.w_int_packed.data_ptr(), self.w_int_packed._version)
+        except RuntimeError:              # a tensor created in inference mode keeps no version counter
+            key = (self.w_int_packed.data_ptr(), None)
+        if self._tiles is None or self._tiles_of != key:
+            self._tiles = weight_tiles(self.w_int_packed)
+            self._tiles_of = key
+        return self._tiles
 
     @classmethod
     def from_weight(cls, weight: torch.Tensor, bias: torch.Tensor = None, use_hadamard: bool = False) -> 'Linear4bit':
@@ -191,6 +231,13 @@ class Linear4bit(nn.Module):
             y += self.bias
         return y
 
+    def forward_tiles(self, a_scale, a_tiles, out=None) -> torch.Tensor:
+        """The same for activations quantised to E2M3 tiles: the GEMM on the FP6 matrix instructions."""
+        y = quest.fused_matmul_dequantize_e2m3(a_tiles, self.w_tiles(), a_scale, self.w_scale, self.weight.size(1), out)
+        if self.bias is not None:
+            y += self.bias
+        return y
+
     def forward(self, x) -> torch.Tensor:
         lead, n = x.shape[:-1], self.weight.size(0)
         rows = x.contiguous().view(-1, x.size(-1))
@@ -201,8 +248,9 @@ class Linear4bit(nn.Module):
                 quest.hadamard128(rows)
             y = torch.zeros(rows.size(0), n, dtype=x.dtype, device=x.device)
         else:
+            m, k = rows.shape
             y = linear_forward(rows, self.w_int_packed, self.w_scale, self.w_add, self.w_meta_e,
-                               use_hadamard=self.use_hadamard)
+                               use_hadamard=self.use_hadamard, w_tiles=self.w_tiles() if prefers_e2m3(m, k, n) else None)
         if self.bias is not None:
             y += self.bias
         return y.view(*lead, n)

@@ -98,6 +98,7 @@ class LlamaMLP(nn.Module):
         self.c_proj = nn.Linear(config.hidden_dim, config.n_embd, bias=False)
         self.w12 = None          # set by quantize_model(..., fuse_gate_up=True): one module for both
         self.glu = None          # enable_swiglu_epilogue(): w12's packed rows in the order the gated-unit GEMM reads
+        self.glu_tiles = None
 
     def enable_swiglu_epilogue(self):
         """A second copy of the fused gate/up weights with the rows interleaved in eights (four gate rows, then the four
@@ -106,6 +107,7 @@ class LlamaMLP(nn.Module):
         w = self.w12
         p = quest.swiglu_interleave_rows(w.w_int_packed.size(0) // 2, device=w.w_int_packed.device)
         self.glu = (w.w_int_packed[p].contiguous(), w.w_scale[p].contiguous(), w.w_add[p].contiguous())
+        self.glu_tiles = None            # the interleaved rows as E2M3 tiles, built on first use
 
     def swiglu_quantized(self, a_scale, a_int_packed, a_int_row_sum):
         """silu(w1 x) * w2 x, (M, hidden), from the codes of x; the gated unit runs in the GEMM's epilogue when that
@@ -117,6 +119,13 @@ class LlamaMLP(nn.Module):
         gate_up = self.w12.forward_quantized(a_scale, a_int_packed, a_int_row_sum)
         h = gate_up.size(-1) // 2
         return F.silu(gate_up[..., :h]) * gate_up[..., h:]
+
+    def swiglu_tiles(self, a_scale, a_tiles):
+        """The same from the E2M3 tiles of x, on the FP6 matrix instructions (needs enable_swiglu_epilogue())."""
+        w_packed, w_scale, _ = self.glu
+        if self.glu_tiles is None:
+            self.glu_tiles = harness.weight_tiles(w_packed)
+        return quest.fused_matmul_dequantize_e2m3(a_tiles, self.glu_tiles, a_scale, w_scale, w_packed.size(1) * 2, swiglu=True)
 
     def forward(self, x):
         if self.w12 is not None:
@@ -187,18 +196,43 @@ class LlamaBlock(nn.Module):
         given, is the previous block's MLP output still to be added to it.  Returns (x, this block's MLP output):
         the caller adds the last one (or hands it to the next block)."""
         b, t, c = x.shape
-        x2 = x.view(b * t, c)
-        if branch is None:
-            q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
+        m = b * t
+        x2 = x.view(m, c)
+        hidden = self.mlp.c_proj.weight.size(1)
+        # each producer writes the operand form its GEMM runs fastest on: E2M3 tiles for the FP6 kernel, or packed
+        # nibbles and row sums for the INT8 kernels (same codes, same output bits either way)
+        if harness.prefers_e2m3(m, c, 3 * c):
+            if branch is None:
+                q = quest.rmsnorm_hadamard_quantize_e2m3(x2, self.ln_1.weight, self.ln_1.eps)
+            else:
+                q = quest.add_rmsnorm_hadamard_quantize_e2m3(x2, branch.view(m, c), self.ln_1.weight, self.ln_1.eps)
+            qkv = self.attn.c_attn.forward_tiles(*q)
         else:
-            q = quest.add_rmsnorm_hadamard_quantize_int4(x2, branch.view(b * t, c), self.ln_1.weight, self.ln_1.eps)
-        att = self.attn.attend(self.attn.c_attn.forward_quantized(*q).view(b, t, 3 * c), freqs_cis)
-        q = quest.add_rmsnorm_hadamard_quantize_int4(x2, att.view(b * t, c), self.ln_2.weight, self.ln_2.eps)
-        if self.mlp.glu is not None:
-            q = quest.hadamard_quantize_int4(self.mlp.swiglu_quantized(*q))
+            if branch is None:
+                q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
+            else:
+                q = quest.add_rmsnorm_hadamard_quantize_int4(x2, branch.view(m, c), self.ln_1.weight, self.ln_1.eps)
+            qkv = self.attn.c_attn.forward_quantized(*q)
+        att = self.attn.attend(qkv.view(b, t, 3 * c), freqs_cis)
+        down_tiles = harness.prefers_e2m3(m, hidden, c)
+        if harness.prefers_e2m3(m, c, 2 * hidden):
+            q = quest.add_rmsnorm_hadamard_quantize_e2m3(x2, att.view(m, c), self.ln_2.weight, self.ln_2.eps)
+            if self.mlp.glu is not None:
+                act = self.mlp.swiglu_tiles(*q)
+                q = quest.hadamard_quantize_e2m3(act) if down_tiles else quest.hadamard_quantize_int4(act)
+            else:
+                gate_up = self.mlp.w12.forward_tiles(*q)
+                q = quest.silu_mul_hadamard_quantize_e2m3(gate_up) if down_tiles else quest.silu_mul_hadamard_quantize_int4(gate_up)
         else:
-            q = quest.silu_mul_hadamard_quantize_int4(self.mlp.w12.forward_quantized(*q))
-        return x, self.mlp.c_proj.forward_quantized(*q).view(b, t, c)
+            q = quest.add_rmsnorm_hadamard_quantize_int4(x2, att.view(m, c), self.ln_2.weight, self.ln_2.eps)
+            if self.mlp.glu is not None:
+                act = self.mlp.swiglu_quantized(*q)
+                q = quest.hadamard_quantize_e2m3(act) if down_tiles else quest.hadamard_quantize_int4(act)
+            else:
+                gate_up = self.mlp.w12.forward_quantized(*q)
+                q = quest.silu_mul_hadamard_quantize_e2m3(gate_up) if down_tiles else quest.silu_mul_hadamard_quantize_int4(gate_up)
+        y = self.mlp.c_proj.forward_tiles(*q) if down_tiles else self.mlp.c_proj.forward_quantized(*q)
+        return x, y.view(b, t, c)
 
 
 class Llama(nn.Module):
@@ -288,10 +322,14 @@ def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, 
             mlp.w1 = _pack(mlp.w1, use_hadamard, noop)
             mlp.w2 = _pack(mlp.w2, use_hadamard, noop)
         mlp.c_proj = _pack(mlp.c_proj, use_hadamard, noop)
-        # the producer-fused kernels exist for the Hadamard variant, rows up to 4096 and the fused gate/up layout
+        # the producer-fused kernels exist for the Hadamard variant, rows up to 32768 and the fused gate/up layout
         block.attn.fused_rope = bool(fuse_producers and not noop)
         block.fuse_producers = bool(fuse_producers and not noop and use_hadamard and fuse_gate_up and
-                                    model.config.n_embd <= 4096 and model.config.hidden_dim <= 4096)
+                                    model.config.n_embd <= 32768 and model.config.hidden_dim <= 32768)
+        if fuse_producers and not noop and not block.fuse_producers:
+            import warnings
+            warnings.warn('quantize_model: fuse_producers asked for, but this configuration (no Hadamard, separate gate / up '
+                          'projections or rows over 32768) has no producer-fused kernels: the blocks run with torch glue')
         if block.fuse_producers and swiglu_epilogue and model.config.hidden_dim % 4 == 0:
             mlp.enable_swiglu_epilogue()
     return model

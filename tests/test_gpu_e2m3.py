@@ -172,3 +172,83 @@ def test_error_codes(quest):
     assert lib.quest_fused_matmul_dequantize_e2m3(fake, fake, fake, fake, fake, 4, 128, 4, 7, null) == -3
     assert lib.quest_int4_to_e2m3_tiles(fake, fake, 4, 100, null) == -2
     assert lib.quest_e2m3_tiles_bytes(4, 100) == 0
+
+
+# --------------------------------------------------------------------------- the activation kernels writing tiles
+def rand_act(m, k, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g) * (torch.rand(m, 1, generator=g) * 4 + 0.05)
+    return x.to(dtype)
+
+
+ACT_SHAPES = [(64, 4096), (33, 1024), (70, 128), (5, 2816), (1, 4096), (257, 256), (40, 11008), (9, 8192), (130, 512), (3, 32768)]
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', ACT_SHAPES)
+def test_activation_tiles_hold_the_packed_codes(quest, dtype, shape):
+    """The tiles written by the fused activation kernel decode to exactly the codes its packed output holds (which the
+    parity tests pin against the oracle), with the same scale, in one launch and in a launch that writes tiles only."""
+    m, k = shape
+    x = rand_act(m, k, dtype, 21).to(DEV)
+    scale, packed, row_sum = quest.hadamard_quantize_int4(x)
+    p2 = torch.empty_like(packed)
+    r2 = torch.empty_like(row_sum)
+    s_both, t_both = quest.hadamard_quantize_e2m3(x, x_int_packed=p2, x_int_row_sum=r2)
+    s_only, t_only = quest.hadamard_quantize_e2m3(x)
+    assert torch.equal(bits(s_both.cpu()), bits(scale.cpu())) and torch.equal(bits(s_only.cpu()), bits(scale.cpu()))
+    assert torch.equal(p2, packed) and torch.equal(r2, row_sum)
+    want = qo.unpack_int4(packed.cpu()).double() + .5
+    assert torch.equal(qo.e2m3_tiles_decode(t_both.cpu(), m, k), want)
+    assert torch.equal(qo.e2m3_tiles_decode(t_only.cpu(), m, k), want)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_activation_tiles_degenerate_rows(quest, dtype):
+    """Zero rows, a NaN, an Inf and huge / tiny magnitudes: the tiles still hold the packed output's codes."""
+    m, k = 8, 512
+    x = rand_act(m, k, dtype, 22)
+    x[1] = 0
+    x[2, 5] = float('nan')
+    x[3, 7] = float('inf')
+    x[4] *= 1e4 if dtype == torch.float16 else 1e30
+    x[5] *= 1e-6 if dtype == torch.float16 else 1e-30
+    x = x.to(DEV)
+    _, packed, _ = quest.hadamard_quantize_int4(x)
+    _, tiles = quest.hadamard_quantize_e2m3(x)
+    assert torch.equal(qo.e2m3_tiles_decode(tiles.cpu(), m, k), qo.unpack_int4(packed.cpu()).double() + .5)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_tiles_fall_back_without_the_matrix_core_transform(quest, dtype):
+    """No transform (hadamard_scale = 0) and the weight-side factor: quantised to packed codes, then converted."""
+    m, k = 40, 384
+    x = rand_act(m, k, dtype, 23).to(DEV)
+    for hs in (0., 2. ** -3.5):
+        _, packed, _ = quest.hadamard_quantize_int4(x, hadamard_scale=hs)
+        _, tiles = quest.hadamard_quantize_e2m3(x, hadamard_scale=hs)
+        assert torch.equal(qo.e2m3_tiles_decode(tiles.cpu(), m, k), qo.unpack_int4(packed.cpu()).double() + .5)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(64, 1024), (33, 4096), (20, 6912), (9, 11008)])
+def test_producer_kernels_write_the_same_tiles(quest, dtype, shape):
+    m, k = shape
+    g = torch.Generator().manual_seed(24)
+    x = rand_act(m, k, dtype, 25).to(DEV)
+    w = (1 + 0.1 * torch.randn(k, generator=g)).to(dtype).to(DEV)
+    s0, p0, _ = quest.rmsnorm_hadamard_quantize_int4(x, w, 1e-5)
+    s1, t1 = quest.rmsnorm_hadamard_quantize_e2m3(x, w, 1e-5)
+    assert torch.equal(bits(s0.cpu()), bits(s1.cpu()))
+    assert torch.equal(qo.e2m3_tiles_decode(t1.cpu(), m, k), qo.unpack_int4(p0.cpu()).double() + .5)
+    br = rand_act(m, k, dtype, 26).to(DEV)
+    xa, xb = x.clone(), x.clone()
+    s0, p0, _ = quest.add_rmsnorm_hadamard_quantize_int4(xa, br, w, 1e-5)
+    s1, t1 = quest.add_rmsnorm_hadamard_quantize_e2m3(xb, br, w, 1e-5)
+    assert torch.equal(bits(xa.cpu()), bits(xb.cpu())) and torch.equal(bits(s0.cpu()), bits(s1.cpu()))
+    assert torch.equal(qo.e2m3_tiles_decode(t1.cpu(), m, k), qo.unpack_int4(p0.cpu()).double() + .5)
+    gu = rand_act(m, 2 * k, dtype, 27).to(DEV)
+    s0, p0, _ = quest.silu_mul_hadamard_quantize_int4(gu)
+    s1, t1 = quest.silu_mul_hadamard_quantize_e2m3(gu)
+    assert torch.equal(bits(s0.cpu()), bits(s1.cpu()))
+    assert torch.equal(qo.e2m3_tiles_decode(t1.cpu(), m, k), qo.unpack_int4(p0.cpu()).double() + .5)

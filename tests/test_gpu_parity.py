@@ -403,7 +403,9 @@ def _ulp_stats(got, want):
     return int(d.max()), float((d != 0).float().mean())
 
 
-PRODUCER_SHAPES = [(160, 1024), (33, 2816), (5, 128), (64, 4096), (7, 256), (9, 512), (12, 2048), (300, 768)]
+PRODUCER_SHAPES = [(160, 1024), (33, 2816), (5, 128), (64, 4096), (7, 256), (9, 512), (12, 2048), (300, 768),
+                   # rows over 4096 (several waves per row): the 1600M model's and Llama-7B's MLP widths among them
+                   (40, 5120), (33, 6912), (17, 8192), (20, 11008), (3, 32768)]
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
@@ -471,12 +473,25 @@ def test_silu_mul_hadamard_quantize(quest, dtype, shape):
     assert torch.equal(bits(scale.cpu()), bits(s2.cpu())) and torch.equal(packed, p2) and torch.equal(row_sum, r2)
 
 
-def test_producers_refuse_long_rows(quest):
-    x = torch.zeros(2, 8192, dtype=torch.bfloat16, device=DEV)
+def test_producers_refuse_rows_over_32768(quest):
+    k = 32768 + 128
+    x = torch.zeros(2, k, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError):
-        quest.rmsnorm_hadamard_quantize_int4(x, torch.ones(8192, dtype=torch.bfloat16, device=DEV), 1e-5)
+        quest.rmsnorm_hadamard_quantize_int4(x, torch.ones(k, dtype=torch.bfloat16, device=DEV), 1e-5)
     with pytest.raises(RuntimeError):
-        quest.silu_mul_hadamard_quantize_int4(torch.zeros(2, 16384, dtype=torch.bfloat16, device=DEV))
+        quest.silu_mul_hadamard_quantize_int4(torch.zeros(2, 2 * k, dtype=torch.bfloat16, device=DEV))
+
+
+def test_llama7b_down_proj_producer(quest):
+    """M = 4096, K = 11008 (the SwiGLU product in front of Llama-7B's down projection): the fused producer equals the
+    producer's own output run through the plain activation kernel, bit for bit."""
+    m, k = 4096, 11008
+    g = torch.Generator(device=DEV).manual_seed(7)
+    gu = torch.randn(m, 2 * k, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    x_act = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+    scale, packed, row_sum = quest.silu_mul_hadamard_quantize_int4(gu, x_act=x_act)
+    s2, p2, r2 = quest.hadamard_quantize_int4(x_act)
+    assert torch.equal(scale.view(torch.int16), s2.view(torch.int16)) and torch.equal(packed, p2) and torch.equal(row_sum, r2)
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
