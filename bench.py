@@ -3,13 +3,16 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step is one W4A4 linear at the Llama-7B gate/up shape (M=4096 tokens, K=4096, N=11008): the
-fused Hadamard + scale + quantise + pack kernel on the fp16 activations, then the packed
-INT4 x INT4 GEMM with the scale epilogue to fp16.  Inputs are synthetic and already resident in
+One step is one W4A4 linear at the Llama-7B gate/up shape (M=4096 tokens, K=4096, N=11008) as
+`harness.linear_forward` runs it at this size: the fused Hadamard + scale + quantise kernel on the fp16
+activations, writing the INT4 codes in the GEMM's operand form (E2M3 tiles), then the INT4 x INT4 GEMM
+on the FP6 matrix instructions with the scale epilogue to fp16 -- the same output bits as the
+packed-nibble INT8 kernels, which are timed beside it.  Inputs are synthetic and already resident in
 HBM; several activation buffers are rotated so that no step finds its input in the Infinity Cache.
 `value` is 2*M*N*K / step time (TOPS of the whole linear, as the reference's published layer times
 are converted).  The JSON line also carries
-  roofline           the GEMM kernel against the INT8 MFMA peak (HIP events around back-to-back launches),
+  roofline           the GEMM kernel against the INT8 MFMA peak, the metric's denominator (HIP events around
+                     back-to-back launches); the FP6 pipe's own peak and the INT8 kernel's figure beside it,
   roofline_quantize  the fused activation kernel at bf16 [8192, 4096] (heavy-tailed input with
                      outlier channels) against the HBM peak,
   decode             the layer at M in {1, 8, 16}: the weight-streaming GEMM alone and with the activation kernel,
@@ -39,14 +42,26 @@ SUSTAIN_MS = 60.0            # launches_ms(..., sustained=True): untimed replays
 EAGER_BATCHES = False        # --eager-batches: time plain launches instead of graph replays
 LAST = {'min_ms': None, 'sustained_ms': None}      # fastest replay of the most recent launches_ms() call
 INT8_MFMA_PEAK_TOPS = 5000.0
+FP6_MFMA_PEAK_TOPS = 10100.0
 
 # HBM bytes per launch from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch),
 # scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
 TRAFFIC_SOURCE = ('constant from a separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this script, summarised in '
                   'profiles/bench_gemm_M4096_K4096_N11008_and_quantize_8192x4096.md; not measured in this run')
-TRAFFIC_GEMM_BYTES = 343078377
+TRAFFIC_GEMM_BYTES = 343078377                 # placeholder until the counter run of this kernel: see TRAFFIC_GEMM_PLAN
 TRAFFIC_QUANTIZE_BYTES = 84236564
+# what quest_e2m3_gemm_plan reported for M=4096 K=4096 N=11008 on 256 compute units when TRAFFIC_GEMM_BYTES was measured: the
+# figure depends on the schedule (which workgroup fetches what), so the line says `traffic_stale` when the plan has changed
+TRAFFIC_GEMM_PLAN = [256, 8, 0, 0, 256, 256, 6, 64]
+
+
+def gemm_plan(lib, m, k, n, dev):
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    plan = (ctypes.c_int * 8)()
+    if lib.quest_e2m3_gemm_plan(m, k, n, cus, plan) != 0:
+        raise RuntimeError('quest_e2m3_gemm_plan failed')
+    return list(plan)
 
 
 def event_pairs(n):
@@ -149,21 +164,27 @@ def bench_linear(quest, _lib, steps, warmup, dev):
     w_packed = ((w_codes[:, 1::2] << 4) | (w_codes[:, ::2] & 0xF)).view(torch.uint8).to(dev)
     w_scale = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
     w_add = (w_codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2).to(dev)
+    w_tiles = quest.int4_to_e2m3_tiles(w_packed)                 # the weights' operand form, made once (as Linear4bit keeps it)
     a_scale = torch.empty(m, 1, dtype=dtype, device=dev)
     a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
     a_row_sum = torch.empty(m, 1, dtype=torch.int32, device=dev)
+    a_tiles = torch.empty(quest.e2m3_tiles_bytes(m, k), dtype=torch.uint8, device=dev)
     out = torch.empty(m, n, dtype=dtype, device=dev)
 
     def step(i, ev=None):
         x = acts[i % n_buf]
         if ev:
             ev[0].record()
-        quest.hadamard_quantize_int4(x, a_scale, a_packed, a_row_sum)
+        quest.hadamard_quantize_e2m3(x, a_scale, a_tiles)
         if ev:
             ev[1].record()
-        quest.fused_matmul_dequantize_int4_int4t_bf16(a_packed, w_packed, a_row_sum, w_add, a_scale, w_scale, out)
+        quest.fused_matmul_dequantize_e2m3(a_tiles, w_tiles, a_scale, w_scale, k, out)
         if ev:
             ev[2].record()
+
+    def step_int8(i):
+        quest.hadamard_quantize_int4(acts[i % n_buf], a_scale, a_packed, a_row_sum)
+        quest.fused_matmul_dequantize_int4_int4t_bf16(a_packed, w_packed, a_row_sum, w_add, a_scale, w_scale, out)
 
     lib = _lib.load()
     for i in range(warmup):
@@ -206,6 +227,8 @@ def bench_linear(quest, _lib, steps, warmup, dev):
     torch.cuda.synchronize()
     ms_per_step_eager = (time.perf_counter() - t0) * 1e3 / steps
     ms_per_step = sorted(step_times_ms)[len(step_times_ms) // 2] if step_times_ms else ms_per_step_eager
+    # the same layer on the packed-nibble path (activation kernel writing nibbles and row sums, INT8 kernel)
+    step_int8_ms = launches_ms(step_int8, steps)
     # the split between the two kernels, from a second pass with events between them (the events cost a few
     # microseconds each, which is why the timed pass above has none)
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
@@ -222,12 +245,23 @@ def bench_linear(quest, _lib, steps, warmup, dev):
     u_row_sum = u_codes.to(torch.int32).sum(-1, keepdim=True).to(torch.int32).to(dev)
     u_scale = (torch.rand(m, 1, generator=g) * 0.09 + 0.01).to(dtype).to(dev)
 
-    def gemm_launcher(codes, row_sum, scale):
+    u_tiles = quest.int4_to_e2m3_tiles(u_packed)
+
+    def gemm_launcher(codes, row_sum, scale):                      # the INT8 kernel on packed nibbles
         args = (_lib.ptr(out), _lib.ptr(codes), _lib.ptr(w_packed), _lib.ptr(row_sum), _lib.ptr(w_add),
                 _lib.ptr(scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype])         # sizes in the ABI's order: M, K, N
 
         def gemm(_):
             if lib.quest_fused_matmul_dequantize_int4_int4t(*args, current_stream()) != 0:
+                raise RuntimeError('GEMM launch failed')
+        return gemm
+
+    def e2m3_launcher(tiles, scale, w=None):                       # the FP6 kernel on E2M3 tiles
+        args = (_lib.ptr(out), _lib.ptr(tiles), _lib.ptr(w_tiles if w is None else w), _lib.ptr(scale), _lib.ptr(w_scale), m, k, n,
+                _lib.DTYPE_CODE[dtype])
+
+        def gemm(_):
+            if lib.quest_fused_matmul_dequantize_e2m3(*args, current_stream()) != 0:
                 raise RuntimeError('GEMM launch failed')
         return gemm
 
@@ -240,21 +274,32 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         if lib.quest_hadamard_quantize_int4(act_ptrs[i % n_buf], *q_tail, current_stream()) != 0:
             raise RuntimeError('activation kernel launch failed')
 
+    t_tail = (_lib.ptr(a_scale), _lib.ptr(a_tiles), None, None, None, k, m, 181. / 2048., _lib.DTYPE_CODE[dtype])
+
+    def quant_tiles_alone(i):
+        if lib.quest_hadamard_quantize_e2m3(act_ptrs[i % n_buf], *t_tail, current_stream()) != 0:
+            raise RuntimeError('activation kernel launch failed')
+
     quant_alone_ms = launches_ms(quant_alone, 100)
-    gemm_quantized_ms = launches_ms(gemm_launcher(a_packed, a_row_sum, a_scale), max(steps, 100))
+    quant_tiles_alone_ms = launches_ms(quant_tiles_alone, 100)
+    step(0)                                                       # a_tiles / a_packed hold the codes of Gaussian activations again
+    step_int8(0)
+    gemm_quantized_ms = launches_ms(e2m3_launcher(a_tiles, a_scale), max(steps, 100))
+    int8_quantized_ms = launches_ms(gemm_launcher(a_packed, a_row_sum, a_scale), max(steps, 100))
     # the same with the weights rotated through 14 copies (315 MB, more than the Infinity Cache holds), as a model
     # with many layers would stream them from HBM
-    w_copies = [w_packed] + [w_packed.clone() for _ in range(13)]
-    u_args = (_lib.ptr(u_row_sum), _lib.ptr(w_add), _lib.ptr(u_scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype])
+    w_copies = [w_tiles] + [w_tiles.clone() for _ in range(9)]    # 10 x 33.8 MB
+    u_args = (_lib.ptr(u_scale), _lib.ptr(w_scale), m, k, n, _lib.DTYPE_CODE[dtype])
     w_ptrs = [_lib.ptr(w) for w in w_copies]
 
     def gemm_rotating(i):
-        if lib.quest_fused_matmul_dequantize_int4_int4t(_lib.ptr(out), _lib.ptr(u_packed), w_ptrs[i % 14], *u_args, current_stream()) != 0:
+        if lib.quest_fused_matmul_dequantize_e2m3(_lib.ptr(out), _lib.ptr(u_tiles), w_ptrs[i % 10], *u_args, current_stream()) != 0:
             raise RuntimeError('GEMM launch failed')
 
-    gemm_rotating_ms = launches_ms(gemm_rotating, 98)
+    gemm_rotating_ms = launches_ms(gemm_rotating, 100)
     del w_copies
-    gemm_ms = launches_ms(gemm_launcher(u_packed, u_row_sum, u_scale), max(steps, 100))
+    int8_gemm_ms = launches_ms(gemm_launcher(u_packed, u_row_sum, u_scale), max(steps, 100))
+    gemm_ms = launches_ms(e2m3_launcher(u_tiles, u_scale), max(steps, 100))
     gemm_min_ms = LAST['min_ms']
     # a yardstick, not part of the path: the vendor library's INT8 GEMM (torch._int_mm -> hipBLASLt) on the same codes as
     # int8, int32 out -- twice the operand bytes, no nibbles to split, no scale arithmetic
@@ -283,6 +328,10 @@ def bench_linear(quest, _lib, steps, warmup, dev):
         'vendor_int8_ms': vendor_int8_ms,
         'quant_ms': quant_ms,
         'quant_alone_ms': quant_alone_ms,
+        'quant_tiles_alone_ms': quant_tiles_alone_ms,
+        'step_int8_ms': step_int8_ms,
+        'int8_gemm_ms': int8_gemm_ms,
+        'int8_quantized_ms': int8_quantized_ms,
     }
 
 
@@ -355,6 +404,7 @@ def bench_decode(_lib, dev, ms=(1, 8, 16)):
     dtype = torch.float16
     code = _lib.DTYPE_CODE[dtype]
     g = torch.Generator(device='cpu').manual_seed(1)
+    work = torch.zeros(16384 + (2 << 20), dtype=torch.uint8, device=dev)       # the split-K workspace, counters zeroed once
     for k, n in [(4096, 4096), (4096, 11008), (11008, 4096)]:
         n_w = max(2, int(600e6 // (n * k // 2)))
         ws = [torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.uint8).to(dev) for _ in range(n_w)]
@@ -375,6 +425,10 @@ def bench_decode(_lib, dev, ms=(1, 8, 16)):
                 if lib.quest_fused_matmul_dequantize_int4_int4t(yp, ap, wp[i % n_w], *g_tail, current_stream()) != 0:
                     raise RuntimeError('GEMM launch failed')
 
+            def gemm_split(i):
+                if lib.quest_fused_matmul_dequantize_int4_int4t_ws(yp, ap, wp[i % n_w], *g_tail, _lib.ptr(work), work.numel(), current_stream()) != 0:
+                    raise RuntimeError('GEMM launch failed')
+
             def layer(i):
                 if lib.quest_hadamard_quantize_int4(*q_args, current_stream()) != 0:
                     raise RuntimeError('activation kernel launch failed')
@@ -383,8 +437,10 @@ def bench_decode(_lib, dev, ms=(1, 8, 16)):
             layer(0)
             gemm_us = launches_ms(gemm, 200, 20) * 1e3
             layer_us = launches_ms(layer, 200, 20) * 1e3
+            split_us = launches_ms(gemm_split, 200, 20) * 1e3 if lib.quest_gemm_workspace_bytes(m, k, n) else None
             wbytes = n * k // 2
             out.append({'M': m, 'K': k, 'N': n, 'gemm_us': round(gemm_us, 2), 'layer_us': round(layer_us, 2),
+                        'gemm_split_k_us': None if split_us is None else round(split_us, 2),
                         'weight_GBs': round(wbytes / gemm_us / 1e3, 1),
                         'frac_hbm': round(wbytes / gemm_us / 1e3 / HBM_PEAK_GBS, 4),
                         'TOPS': round(2.0 * m * n * k / gemm_us / 1e6, 1)})
@@ -568,14 +624,24 @@ def main():
     if cpu is not None:
         cpu['gpu_same_workload'] = bench_small_layer_gpu(quest, dev)
 
+    ops_gemm = 2.0 * 4096 * 4096 * 11008
+    plan = gemm_plan(_lib.load(), 4096, 4096, 11008, dev)
+    int8_tops = ops_gemm / (lin['int8_gemm_ms'] * 1e-3) / 1e12
     roofline = {'bound': 'mfma', 'achieved': lin['gemm_tops'], 'peak': INT8_MFMA_PEAK_TOPS, 'unit': 'TOP/s',
-                'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS, 'traffic': TRAFFIC_GEMM_BYTES, 'traffic_source': TRAFFIC_SOURCE,
-                'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
+                'frac': lin['gemm_tops'] / INT8_MFMA_PEAK_TOPS,
+                'peak_is': 'INT8 MFMA dense, the peak the metric is stated against; the kernel runs the same INT4 x INT4 products '
+                           'on the FP6 (E2M3) matrix instructions, whose own dense peak is 10.1 PFLOP/s: frac_of_fp6_peak',
+                'frac_of_fp6_peak': lin['gemm_tops'] / FP6_MFMA_PEAK_TOPS,
+                'traffic': TRAFFIC_GEMM_BYTES, 'traffic_source': TRAFFIC_SOURCE, 'traffic_plan': TRAFFIC_GEMM_PLAN, 'plan': plan,
+                'traffic_stale': plan != TRAFFIC_GEMM_PLAN,
+                'kernel': 'gemm_e2m3_kernel', 'us_per_launch': lin['gemm_ms'] * 1e3,
                 'us_per_launch_min': lin['gemm_min_ms'] * 1e3,
                 'us_per_launch_weights_from_hbm': lin['gemm_rotating_weights_ms'] * 1e3,
+                'int8_kernel_same_codes': {'kernel': 'gemm_w4a4_big_kernel', 'us_per_launch': lin['int8_gemm_ms'] * 1e3,
+                                           'achieved': int8_tops, 'frac': int8_tops / INT8_MFMA_PEAK_TOPS},
                 'vendor_int8_gemm_same_shape_us': None if lin['vendor_int8_ms'] is None else lin['vendor_int8_ms'] * 1e3,
-                'algorithmic_ops': 2.0 * 4096 * 4096 * 11008,
-                'workload': 'uniform random INT4 codes on both sides, M=4096 K=4096 N=11008, fp16 out'}
+                'algorithmic_ops': ops_gemm,
+                'workload': 'uniform random INT4 codes on both sides (as E2M3 tiles), M=4096 K=4096 N=11008, fp16 out'}
     line = {
         'metric': 'INT4-GEMM TOPS + quantize GB/s at Llama-7B layer shapes, % MI355X roofline',
         'value': lin['tops'], 'unit': 'TOPS', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -584,15 +650,23 @@ def main():
                       f"{lin['untimed_replays']} untimed replays (60 ms: the clocks settle); median of five such timings, all in "
                       "ms_per_step_each; the eager figure beside it",
         'ms_per_step_each': lin['ms_per_step_each'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'int8', 'data': 'synthetic',
+        'dtype': 'fp6 (E2M3 products of INT4 codes, fp32 accumulation: exact)', 'data': 'synthetic',
         'config': {'workload': 'W4A4 linear, Llama-7B gate/up: fp16 activations [4096,4096] -> fused '
-                               'Hadamard-quantize-pack -> packed INT4 GEMM [4096,4096]x[11008,4096]^T -> fp16 [4096,11008]',
+                               'Hadamard-quantize (INT4 codes as E2M3 tiles) -> INT4 x INT4 GEMM [4096,4096]x[11008,4096]^T on the FP6 '
+                               'matrix instructions -> fp16 [4096,11008]',
                    'M': 4096, 'K': 4096, 'N': 11008},
         'gemm_tops': lin['gemm_tops'], 'gemm_us_in_step': lin['gemm_in_step_ms'] * 1e3,
         'gemm_tops_on_quantized_activations': 2.0 * 4096 * 4096 * 11008 / (lin['gemm_quantized_acts_ms'] * 1e-3) / 1e12,
+        'packed_nibble_path': {'what': 'the same layer through the activation kernel writing nibbles and the INT8 kernels (same output bits)',
+                               'us_per_step': lin['step_int8_ms'] * 1e3,
+                               'gemm_us_on_quantized_activations': lin['int8_quantized_ms'] * 1e3},
         'quantize_us_in_step': lin['quant_ms'] * 1e3,
         'quantize_GBs': rq['achieved'],
-        'quantize_in_step_shape': {'workload': 'fp16 [4096,4096] (the step\'s own activation kernel), graph of 100 bare launches',
+        'quantize_tiles_in_step_shape': {'workload': 'fp16 [4096,4096] -> E2M3 tiles + scales (the step\'s own activation kernel), graph of 100 bare launches',
+                                         'us_per_launch': lin['quant_tiles_alone_ms'] * 1e3,
+                                         'GBs': (4096 * 4096 * 2.75 + 4096 * 2) / (lin['quant_tiles_alone_ms'] * 1e-3) / 1e9,
+                                         'frac_hbm': (4096 * 4096 * 2.75 + 4096 * 2) / (lin['quant_tiles_alone_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        'quantize_in_step_shape': {'workload': 'fp16 [4096,4096] -> packed nibbles, scales, row sums (the packed path\'s activation kernel), graph of 100 bare launches',
                                    'us_per_launch': lin['quant_alone_ms'] * 1e3,
                                    'GBs': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9,
                                    'frac_hbm': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS},

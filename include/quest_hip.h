@@ -89,6 +89,25 @@ int quest_fused_matmul_dequantize_int4_int4t(void *mat_d, const uint8_t *mat_a, 
                                              int size_m, int size_k, int size_n, int dtype, void *stream);
 
 /*
+ * quest_fused_matmul_dequantize_int4_int4t with a caller-owned workspace, which lets a handful of tokens
+ * (size_m <= 16: the decode shapes) split K across workgroups: every slice leaves its partial int32 tile in the
+ * workspace and the workgroup that arrives last (a counter per channel tile, no atomics on the result) adds them --
+ * integers, so the result does not depend on the order -- and applies the epilogue.  Same outputs bit for bit.
+ * The reference passes no workspace to its CUTLASS GEMM (quest/matmul_kernel.cu:55: nullptr) and runs no split-K.
+ * workspace: quest_gemm_workspace_bytes(size_m, size_k, size_n) bytes (0: this shape does not use one), 256-byte
+ * aligned; its first 16 KiB (the counters) must be zero before the first call and are zero again after every call,
+ * so one zero-initialised buffer serves any number of calls -- but calls that may overlap in time (different
+ * streams) need a workspace each.  Shapes that do not split, or a workspace that is NULL or too small, run exactly as
+ * quest_fused_matmul_dequantize_int4_int4t.
+ */
+size_t quest_gemm_workspace_bytes(int size_m, int size_k, int size_n);
+int quest_fused_matmul_dequantize_int4_int4t_ws(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                const void *vec_a_mul, const void *vec_b_mul, int size_m, int size_k,
+                                                int size_n, int dtype, void *workspace, size_t workspace_bytes,
+                                                void *stream);
+
+/*
  * y = block-128 Walsh-Hadamard transform of every row of x along K, fp32 butterflies, * had_scale,
  * one rounding to dtype.  had_scale = 181/2048 reproduces F.linear(x.view(-1,128), HADAMARD_MATRIX)
  * (benchmarks/utils.py:17,89-90: the matrix entries are bf16(2^-3.5) = 181/2048); had_scale = 2^-3.5
@@ -126,6 +145,11 @@ int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t *x_int_pack
  */
 #define QUEST_SCALE_GAUSSIAN 0
 #define QUEST_SCALE_ABSMAX 1
+/* OR-ed into scale_rule: scale and codes from the transform's fp32 output and the unrounded scale (fp32 butterflies, any
+ * had_scale), the arithmetic of the reference's evaluation-side fake quantiser (src/eval_hswag.py:201-214), instead of
+ * from the dtype-rounded tensor that linear_forward materialises (benchmarks/utils.py:89-100).  The stored scale is still
+ * rounded to dtype.  For comparing a packed model with its fake-quantised original; not bit-pinned. */
+#define QUEST_QUANT_FROM_FP32 4
 int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
                                       void *x_had, int group_size, int batch_size, float had_scale,
                                       int scale_rule, int dtype, void *stream);
@@ -224,6 +248,15 @@ int quest_int4_to_e2m3_tiles(void *tiles, const uint8_t *x_int_packed, int rows,
 int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles, const void *vec_a_mul,
                                        const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
                                        void *stream);
+
+/*
+ * Diagnostic (host only, nothing is launched): how quest_fused_matmul_dequantize_e2m3 divides a shape among the
+ * workgroups of a device with `cus` compute units.  plan[0..7] = workgroups, scheduling groups (one per XCD when 8),
+ * tiles per token tile when every workgroup gets exactly one (else 0), whether the groups divide the token tiles (1) or
+ * the channel units (0), tile rows, tile channels at most, LDS slots, k per slot.  A measured figure that depends on
+ * the schedule (HBM traffic per launch) is only valid while this plan is the one it was measured under.
+ */
+int quest_e2m3_gemm_plan(int size_m, int size_k, int size_n, int cus, int *plan);
 
 /* The same with the SwiGLU epilogue of quest_fused_matmul_dequantize_swiglu_int4_int4t (b_tiles and vec_b_mul in its
  * interleaved row order); mat_d is (size_m, size_n / 2). */

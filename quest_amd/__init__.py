@@ -31,6 +31,9 @@ from .api import (  # noqa: F401
     rmsnorm_hadamard_quantize_e2m3,
     add_rmsnorm_hadamard_quantize_e2m3,
     silu_mul_hadamard_quantize_e2m3,
+    GEMM_WORKSPACE_MAX_BYTES,
+    gemm_workspace,
+    gemm_workspace_bytes,
 )
 
 __version__ = '0.1.0'

@@ -36,17 +36,21 @@ SIGNATURES = {
     'quest_hadamard_quantize_int4_rule': [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
     'quest_rope_interleaved': [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     'quest_silu_mul_hadamard_quantize_int4': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
+    'quest_gemm_workspace_bytes': [_i, _i, _i],
+    'quest_fused_matmul_dequantize_int4_int4t_ws': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp],
     'quest_e2m3_tiles_bytes': [_i, _i],
     'quest_int4_to_e2m3_tiles': [_vp, _vp, _i, _i, _vp],
     'quest_fused_matmul_dequantize_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     'quest_fused_matmul_dequantize_swiglu_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    'quest_e2m3_gemm_plan': [_i, _i, _i, _i, _vp],
     'quest_hadamard_quantize_e2m3': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_rmsnorm_hadamard_quantize_e2m3': [_vp, _vp, _f, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_add_rmsnorm_hadamard_quantize_e2m3': [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_silu_mul_hadamard_quantize_e2m3': [_vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
 }
 # entry points that do not return an int status
-_RESTYPES = {'quest_status_string': ctypes.c_char_p, 'quest_e2m3_tiles_bytes': ctypes.c_size_t}
+_RESTYPES = {'quest_status_string': ctypes.c_char_p, 'quest_e2m3_tiles_bytes': ctypes.c_size_t,
+             'quest_gemm_workspace_bytes': ctypes.c_size_t}
 
 _lib = None
 

@@ -25,8 +25,12 @@ def fused_matmul_dequantize_int4_int4t_bf16(
         vec_a_mul: torch.Tensor,
         vec_b_mul: torch.Tensor,
         out: torch.Tensor = None,
+        workspace: torch.Tensor = None,
 ) -> torch.Tensor:
-    """gemm-quest/quest/__init__.py:6-20.  The output dtype follows vec_a_mul (bf16 or fp16)."""
+    """gemm-quest/quest/__init__.py:6-20.  The output dtype follows vec_a_mul (bf16 or fp16).
+
+    `workspace` (not in the reference): a uint8 tensor from `gemm_workspace`, which lets up to 16 tokens split K across
+    workgroups; the result is the same bit for bit.  One workspace serves any number of calls on one stream."""
     if out is None:
         out = torch.empty(mat_a.size(0), mat_b.size(0), dtype=vec_a_mul.dtype, device=mat_a.device)
     assert mat_a.dtype == torch.uint8 and mat_b.dtype == torch.uint8 and vec_a_add.dtype == torch.int32 and vec_b_add.dtype == torch.int32
@@ -37,11 +41,31 @@ def fused_matmul_dequantize_int4_int4t_bf16(
     assert out.size(0) == mat_a.size(0) and out.size(1) == mat_b.size(0)
     dev = require_gpu(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, out)
     with torch.cuda.device(dev):
-        check(_lib.load().quest_fused_matmul_dequantize_int4_int4t(
-            ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
-            mat_a.size(0), mat_b.size(1) * 2, mat_b.size(0), DTYPE_CODE[out.dtype], stream_of(out)),
-            'fused_matmul_dequantize_int4_int4t')
+        if workspace is not None:
+            assert workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.device == out.device
+            check(_lib.load().quest_fused_matmul_dequantize_int4_int4t_ws(
+                ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
+                mat_a.size(0), mat_b.size(1) * 2, mat_b.size(0), DTYPE_CODE[out.dtype], ptr(workspace), workspace.numel(),
+                stream_of(out)), 'fused_matmul_dequantize_int4_int4t_ws')
+        else:
+            check(_lib.load().quest_fused_matmul_dequantize_int4_int4t(
+                ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
+                mat_a.size(0), mat_b.size(1) * 2, mat_b.size(0), DTYPE_CODE[out.dtype], stream_of(out)),
+                'fused_matmul_dequantize_int4_int4t')
     return out
+
+
+GEMM_WORKSPACE_MAX_BYTES = 16384 + (2 << 20)         # the most quest_gemm_workspace_bytes returns for any shape
+
+
+def gemm_workspace_bytes(size_m: int, size_k: int, size_n: int) -> int:
+    """Bytes of workspace the split-K decode GEMM uses for this shape (0: it does not split)."""
+    return int(_lib.load().quest_gemm_workspace_bytes(size_m, size_k, size_n))
+
+
+def gemm_workspace(device, nbytes: int = GEMM_WORKSPACE_MAX_BYTES) -> torch.Tensor:
+    """A zeroed workspace for `fused_matmul_dequantize_int4_int4t(..., workspace=)`; every call leaves it reusable."""
+    return torch.zeros(nbytes, dtype=torch.uint8, device=device)
 
 
 # the same kernel serves both 16-bit float types
@@ -210,14 +234,17 @@ def hadamard_quantize_int4(
         x_had: torch.Tensor = None,
         hadamard_scale: float = HADAMARD_ENTRY,
         scale_rule: str = 'gaussian',
+        from_fp32: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """One pass over x: block-128 Hadamard (skipped when hadamard_scale == 0), Gaussian-clip scale,
     INT4 codes packed two per byte, and their row sums -- the three launches of
     gemm-quest/benchmarks/utils.py:89-100 in one.  x_had, if given, receives the transformed
     activations the codes were computed from.  scale_rule: 'gaussian' (the reference's RMS rule) or 'absmax'
-    (scale = max|x| / 7.5 + 1e-8).  Returns (scale, x_int_packed, x_int_row_sum)."""
+    (scale = max|x| / 7.5 + 1e-8).  from_fp32: scale and codes from the transform's fp32 output (the arithmetic of the
+    reference's evaluation-side fake quantiser, src/eval_hswag.py:201-214) instead of from the dtype-rounded tensor.
+    Returns (scale, x_int_packed, x_int_row_sum)."""
     m, k = x.shape
-    rule = {'gaussian': 0, 'absmax': 1}[scale_rule]
+    rule = {'gaussian': 0, 'absmax': 1}[scale_rule] | (4 if from_fp32 else 0)
     if scale is None:
         scale = torch.empty(m, 1, dtype=x.dtype, device=x.device)
     if x_int_packed is None:

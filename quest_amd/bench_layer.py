@@ -9,10 +9,13 @@ buffer, plain launches and a replayed HIP graph, the smaller of the two):
   int4      harness.linear_forward(..., use_hadamard=False)             (bench_layer.py:37-42)
   int4_had  harness.linear_forward(..., use_hadamard=True)              (bench_layer.py:43-48)
 
-on operands that are allocated but never initialised, exactly as the reference does
-(bench_layer.py:22-29): run time of these kernels does not depend on the values except through the
-power the matrix cores draw, which makes these figures slightly optimistic next to bench.py's
-random-code GEMM.
+The reference leaves its operands uninitialised (bench_layer.py:22-29).  Here the activation pool is filled with
+Gaussian values, the weight codes are random and the weight scales lie in [0.01, 0.1]: the run time of these kernels
+does depend on the values -- the activation kernel takes a slower, clamping path for rows whose scale is zero, Inf or
+NaN, which garbage memory can produce, and the matrix cores' clock follows the power that the operands' bit patterns
+draw -- so finite, realistic data is what keeps the figures honest.  Layer i + 1 still quantises what layer i wrote
+(one buffer serves as input and output, as in the reference), which stays finite.  With enough tokens the INT4 columns
+run the FP6 matrix-core kernel on E2M3 tiles (`harness.prefers_e2m3`), otherwise the INT8 kernels on packed nibbles.
 
     python -m quest_amd.bench_layer [--quick] [--json out.json] [--markdown out.md]
 
@@ -48,10 +51,14 @@ RTX4090_US = {
 def time_layer(n: int, k: int, m: int, dtype=torch.bfloat16, device=None, n_layers: int = 20, n_warmup: int = 3):
     """Seconds per layer for (dense, int4, int4_had) at one shape."""
     device = torch.device('cuda') if device is None else device
-    weight = torch.empty(n, k, dtype=dtype, device=device)
-    w_scale = torch.empty(n, 1, dtype=dtype, device=device)
-    w_int_packed = torch.empty(n, k // 2, dtype=torch.uint8, device=device)
-    w_add = torch.empty(n, 1, dtype=torch.int32, device=device)
+    g = torch.Generator(device=device).manual_seed(0)
+    weight = torch.randn(n, k, dtype=dtype, device=device, generator=g) * 0.02
+    w_scale = (torch.rand(n, 1, device=device, generator=g) * 0.09 + 0.01).to(dtype)
+    w_int_packed = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=device, generator=g)
+    w_add = (harness.unpack_int4(w_int_packed).to(torch.int32).sum(-1, keepdim=True) + k // 2).to(torch.int32)
+    use_tiles = harness.prefers_e2m3(m, k, n)
+    w_tiles = harness.weight_tiles(w_int_packed) if use_tiles else None
+    a_tiles = torch.empty(harness.quest.e2m3_tiles_bytes(m, k), dtype=torch.uint8, device=device) if use_tiles else None
     a_scale = torch.empty(m, 1, dtype=dtype, device=device)
     a_int_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=device)
     a_int_row_sum = torch.empty(m, 1, dtype=torch.int32, device=device)
@@ -63,7 +70,7 @@ def time_layer(n: int, k: int, m: int, dtype=torch.bfloat16, device=None, n_laye
         def layer(a_in, a_out):
             harness.linear_forward(activation=a_in, w_int_packed=w_int_packed, w_scale=w_scale, w_add=w_add, w_meta_e=None,
                                    out=a_out, _a_scale=a_scale, _a_int_packed=a_int_packed, _a_int_row_sum=a_int_row_sum,
-                                   use_hadamard=use_hadamard)
+                                   use_hadamard=use_hadamard, w_tiles=w_tiles, _a_tiles=a_tiles)
         return layer
 
     kw = dict(dtype=dtype, device=device, n_layers=n_layers, n_warmup=n_warmup)

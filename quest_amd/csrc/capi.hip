@@ -1,7 +1,7 @@
 // Version and status text of libquest_hip.
 #include "common.h"
 
-extern "C" int quest_version(void) { return 100; }
+extern "C" int quest_version(void) { return 101; }
 
 extern "C" const char *quest_status_string(int status) {
     switch (status) {

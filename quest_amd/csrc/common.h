@@ -297,6 +297,12 @@ enum { OUT_BF16 = 0, OUT_FP16 = 1, OUT_INT32 = 2 };
 int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                        const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);
 
+// ... and its split-K form for M <= 16 with a workspace (see gemm_decode.hip); gemm_decode_workspace_bytes is what it needs
+int launch_gemm_decode_splitk(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                              const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, void *workspace,
+                              size_t workspace_bytes, hipStream_t st);
+size_t gemm_decode_workspace_bytes(int K, int N);
+
 // hadamard_mfma.hip: the matrix-core fused activation kernel, optionally with the producer of the activation in
 // front (pre: 0 none, 1 RMSNorm, 2 SiLU(gate) * up); QUEST_ERR_UNSUPPORTED when it does not apply
 int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, float eps, void *scale, uint8_t *packed,
@@ -305,6 +311,10 @@ int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, fl
 
 inline int check_dtype(int dtype) { return dtype == QUEST_DTYPE_BF16 || dtype == QUEST_DTYPE_FP16; }
 inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+// HIP keeps the last error until someone reads it.  An entry point judges its own launches by that error, so whatever an
+// earlier call left behind (a failed call of the caller's in this thread, a failed device query in here) is read and
+// dropped first: forget_stale_error() before the first launch of an entry point, launch_status() after the last.
+inline void forget_stale_error() { (void)hipGetLastError(); }
 inline int launch_status() { return hipGetLastError() == hipSuccess ? QUEST_OK : QUEST_ERR_LAUNCH; }
 
 }  // namespace quest

@@ -99,6 +99,7 @@ using namespace quest;
 
 extern "C" int quest_matmul_int4_int4t_int32(int32_t *mat_c, const uint8_t *mat_a, const uint8_t *mat_b, int size_m,
                                              int size_k, int size_n, void *stream) {
+    forget_stale_error();
     const int rc = gemm_check(mat_c, mat_a, mat_b, size_m, size_k, size_n);
     if (rc != QUEST_OK) return rc;
     return gemm_launch(OUT_INT32, mat_c, mat_a, mat_b, nullptr, nullptr, nullptr, nullptr, size_m, size_k, size_n,
@@ -109,6 +110,7 @@ extern "C" int quest_fused_matmul_dequantize_int4_int4t(void *mat_d, const uint8
                                                         const int32_t *vec_a_add, const int32_t *vec_b_add,
                                                         const void *vec_a_mul, const void *vec_b_mul, int size_m,
                                                         int size_k, int size_n, int dtype, void *stream) {
+    forget_stale_error();
     const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
     if (rc != QUEST_OK) return rc;
     if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul) return QUEST_ERR_NULL_POINTER;
@@ -117,10 +119,34 @@ extern "C" int quest_fused_matmul_dequantize_int4_int4t(void *mat_d, const uint8
                        vec_b_mul, size_m, size_k, size_n, (hipStream_t)stream);
 }
 
+extern "C" size_t quest_gemm_workspace_bytes(int size_m, int size_k, int size_n) {
+    if (size_m <= 0 || size_k <= 0 || size_n <= 0 || size_m > 16 || (size_k & 127) || size_n > 65536) return 0;
+    return gemm_decode_workspace_bytes(size_k, size_n);
+}
+
+extern "C" int quest_fused_matmul_dequantize_int4_int4t_ws(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                           const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                           const void *vec_a_mul, const void *vec_b_mul, int size_m,
+                                                           int size_k, int size_n, int dtype, void *workspace,
+                                                           size_t workspace_bytes, void *stream) {
+    forget_stale_error();
+    const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
+    if (rc != QUEST_OK) return rc;
+    if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    const int out_kind = dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16;
+    const int split = launch_gemm_decode_splitk(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m,
+                                                size_k, size_n, workspace, workspace_bytes, (hipStream_t)stream);
+    if (split != QUEST_ERR_UNSUPPORTED) return split;
+    return gemm_launch(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m, size_k, size_n,
+                       (hipStream_t)stream);
+}
+
 extern "C" int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
                                                                const int32_t *vec_a_add, const int32_t *vec_b_add,
                                                                const void *vec_a_mul, const void *vec_b_mul, int size_m,
                                                                int size_k, int size_n, int dtype, void *stream) {
+    forget_stale_error();
     const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
     if (rc != QUEST_OK) return rc;
     if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul) return QUEST_ERR_NULL_POINTER;

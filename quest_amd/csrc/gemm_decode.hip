@@ -171,6 +171,138 @@ gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
     }
 }
 
+// ---- the same for M <= 16 with K split across workgroups --------------------------------------------------------------
+// A workgroup of four waves multiplies 16 channels by one of S slices of K and leaves its partial int32 tile (1 KiB) in
+// the caller's workspace; a counter per channel tile tells the workgroup that arrives last, which adds the S partial
+// tiles (integers: any order gives the same sum), applies the epilogue, stores, and puts the counter back to zero.  No
+// atomic touches the result.  S times the workgroups of the kernel above for the same bytes: shorter dependent chains
+// per wave for long rows.  Workspace: ceil(N / 16) counters (zero before the first use, zero again after every launch),
+// then, from byte kSplitPartialsAt on, ceil(N / 16) x S tiles of 256 ints.
+constexpr int kSplitWaves = 4;
+constexpr size_t kSplitPartialsAt = 16384;          // room for 4096 counters: N <= 65536
+
+template <int OUT>
+__global__ void __launch_bounds__(64 * kSplitWaves, 8)
+gemm_w4a4_decode_splitk_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
+                               const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
+                               const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul, int M, int N, int K,
+                               int *__restrict__ counters, int *__restrict__ partials) {
+    __shared__ __attribute__((aligned(16))) int red[kSplitWaves][64][4];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int row_b = K >> 1;
+    const int tile = blockIdx.x;
+    const int ch0 = tile * kChannels;
+    const int splits = gridDim.y;
+    const int n_chunks = (row_b + kChunkB - 1) / kChunkB;
+    const int c_lo = (int)(((long)n_chunks * blockIdx.y) / splits);
+    const int c_hi = (int)(((long)n_chunks * (blockIdx.y + 1)) / splits);
+
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)wgt, 0, (int)((long)N * row_b), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ar = __builtin_amdgcn_make_buffer_rsrc((void *)act, 0, (int)((long)M * row_b), 0x00020000);
+    const uint32_t dead = 0x80000000u;
+    const uint32_t w_off = (ch0 + r < N) ? (uint32_t)((ch0 + r) * row_b + g * 16) : dead;
+    const uint32_t a_off = (r < M) ? (uint32_t)(r * row_b + g * 16) : dead;
+
+    v4i acc = v4i{0, 0, 0, 0};
+    for (int c0 = c_lo + wave; c0 < c_hi; c0 += kSplitWaves * kBatch) {
+        v4i wq[kBatch][2], aq[kBatch][2];
+#pragma unroll
+        for (int i = 0; i < kBatch; i++) {
+            const int c = c0 + i * kSplitWaves;
+            const int cb = c * kChunkB;
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                const bool in_row = c < c_hi && cb + 64 * hlf < row_b;
+                const uint32_t shift = (uint32_t)(cb + 64 * hlf);
+                wq[i][hlf] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, (int)(in_row ? w_off + shift : dead), 0, 0));
+                aq[i][hlf] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, (int)(in_row ? a_off + shift : dead), 0, 0));
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < kBatch; i++)
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                v4i we, wo, ae, ao;
+                split16(wq[i][hlf], we, wo);
+                split16(aq[i][hlf], ae, ao);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(we, ae, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wo, ao, acc, 0, 0, 0);
+            }
+    }
+
+    // ---- the workgroup's partial tile: the four waves meet in LDS, wave 0 carries it on
+    *reinterpret_cast<v4i *>(&red[wave][lane][0]) = acc;
+    __syncthreads();
+    if (wave != 0) return;
+    v4i sum = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; w++) {
+        const v4i p = *reinterpret_cast<const v4i *>(&red[w][lane][0]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum[e] += p[e];
+    }
+    if (splits > 1) {
+        // publish, count, and let the last arriver gather.  The fences are device-wide releases / acquires: the slices of
+        // one channel tile may run on different XCDs, whose L2 caches do not see each other's lines otherwise.
+        int *mine = partials + ((size_t)tile * splits + blockIdx.y) * 256;
+        *reinterpret_cast<v4i *>(mine + lane * 4) = sum;
+        __threadfence();
+        int arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counters + tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (__builtin_amdgcn_readfirstlane(arrived) != splits - 1) return;
+        __threadfence();
+        sum = v4i{0, 0, 0, 0};
+        for (int sl = 0; sl < splits; sl++) {
+            const v4i p = *reinterpret_cast<const v4i *>(partials + ((size_t)tile * splits + sl) * 256 + lane * 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) sum[e] += p[e];
+        }
+        if (lane == 0) __hip_atomic_store(counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     // ready for the next launch
+    }
+
+    const int tok = r;
+    const int ch = ch0 + 4 * g;
+    if (tok >= M || ch >= N) return;
+    int c[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) c[e] = sum[e] >> 8;      // exact: every product carries 16 * 16
+    const size_t o = (size_t)tok * N + ch;
+    if constexpr (OUT == OUT_INT32) {
+        int32_t *dst = reinterpret_cast<int32_t *>(out) + o;
+        if ((N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+            *reinterpret_cast<int4 *>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (ch + e < N) dst[e] = c[e];
+        }
+    } else {
+        const int t_add = a_add[tok];
+        const float t_half_mul = __fmul_rn(0.5f, to_f32<OUT>(a_mul[tok]));
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int che = min(ch + e, N - 1);
+            const float lhs = (float)(c[e] * 2 + t_add + b_add[che]);
+            const float rhs = __fmul_rn(t_half_mul, to_f32<OUT>(b_mul[che]));
+            h[e] = from_f32<OUT>(__fmul_rn(lhs, rhs));
+        }
+        uint16_t *dst = reinterpret_cast<uint16_t *>(out) + o;
+        if ((N & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0) {
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (ch + e < N) dst[e] = (uint16_t)h[e];
+        }
+    }
+}
+
 template <int OUT, int TM>
 static void launch_tm(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
                       const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
@@ -188,7 +320,48 @@ static int launch_out(void *out, const uint8_t *a, const uint8_t *b, const int32
     return launch_status();
 }
 
+// How many slices of K pay for M <= 16 tokens: enough workgroups to fill the chip several times over, at least two
+// 256-k chunks per wave of a slice.
+static int decode_splits(int K, int N) {
+    const int tiles = (N + kChannels - 1) / kChannels;
+    const int n_chunks = ((K >> 1) + kChunkB - 1) / kChunkB;
+    int s = 1;
+    while (s < 8 && tiles * s * 2 <= 2048 && n_chunks / (s * 2) >= kSplitWaves) s *= 2;
+    return s;
+}
+
 }  // namespace decode
+
+size_t gemm_decode_workspace_bytes(int K, int N) {
+    const int tiles = (N + decode::kChannels - 1) / decode::kChannels;
+    const int splits = decode::decode_splits(K, N);
+    return splits < 2 ? 0 : decode::kSplitPartialsAt + (size_t)tiles * splits * 256 * sizeof(int);
+}
+
+// The split-K form: M <= 16, K % 128 == 0, N <= 65536, a workspace of gemm_decode_workspace_bytes whose counters are zero.
+// QUEST_ERR_UNSUPPORTED when it does not apply or would not split (the caller then takes the kernel above).
+int launch_gemm_decode_splitk(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                              const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, void *workspace,
+                              size_t workspace_bytes, hipStream_t st) {
+    if (M > 16 || (K & 127) != 0 || N > 65536 || !aligned(a, 16) || !aligned(b, 16) || !aligned(workspace, 256)) return QUEST_ERR_UNSUPPORTED;
+    const int splits = decode::decode_splits(K, N);
+    if (splits < 2 || workspace == nullptr || workspace_bytes < gemm_decode_workspace_bytes(K, N)) return QUEST_ERR_UNSUPPORTED;
+    const dim3 grid((N + decode::kChannels - 1) / decode::kChannels, splits), block(64 * decode::kSplitWaves);
+    int *counters = (int *)workspace;
+    int *partials = (int *)((uint8_t *)workspace + decode::kSplitPartialsAt);
+    switch (out_kind) {
+        case OUT_BF16:
+            decode::gemm_w4a4_decode_splitk_kernel<OUT_BF16><<<grid, block, 0, st>>>(out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, counters, partials);
+            break;
+        case OUT_FP16:
+            decode::gemm_w4a4_decode_splitk_kernel<OUT_FP16><<<grid, block, 0, st>>>(out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, counters, partials);
+            break;
+        default:
+            decode::gemm_w4a4_decode_splitk_kernel<OUT_INT32><<<grid, block, 0, st>>>(out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, counters, partials);
+            break;
+    }
+    return launch_status();
+}
 
 // The weight-streaming kernel applies to M <= 128 and K a multiple of 128 (whole 64-byte pieces); QUEST_ERR_UNSUPPORTED otherwise.
 int launch_gemm_decode(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,

@@ -468,6 +468,7 @@ extern "C" size_t quest_e2m3_tiles_bytes(int rows, int size_k) {
 }
 
 extern "C" int quest_int4_to_e2m3_tiles(void *tiles, const uint8_t *x_int_packed, int rows, int size_k, void *stream) {
+    forget_stale_error();
     if (!tiles || !x_int_packed) return QUEST_ERR_NULL_POINTER;
     if (rows <= 0 || size_k <= 0 || (size_k & 63)) return QUEST_ERR_BAD_SHAPE;
     if (!aligned(tiles, 16) || !aligned(x_int_packed, 16)) return QUEST_ERR_ALIGNMENT;
@@ -481,15 +482,27 @@ extern "C" int quest_int4_to_e2m3_tiles(void *tiles, const uint8_t *x_int_packed
 extern "C" int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles, const void *vec_a_mul,
                                                   const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
                                                   void *stream) {
+    forget_stale_error();
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
     return launch_e2m3<false>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                               size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
 }
 
+extern "C" int quest_e2m3_gemm_plan(int size_m, int size_k, int size_n, int cus, int *plan) {
+    if (!plan) return QUEST_ERR_NULL_POINTER;
+    if (size_m <= 0 || size_n <= 0 || size_k <= 0 || (size_k & 127) || cus <= 0) return QUEST_ERR_BAD_SHAPE;
+    long grid = 0;
+    const Schedule sch = make_schedule(size_m, size_n, e2m3::kMaxUnits, 1, cus, &grid);
+    const int v[8] = {(int)grid, sch.groups, sch.row_tiles, sch.by_tokens, e2m3::kRows, 32 * e2m3::kMaxUnits, e2m3::kStages, 64};
+    for (int i = 0; i < 8; i++) plan[i] = v[i];
+    return QUEST_OK;
+}
+
 extern "C" int quest_fused_matmul_dequantize_swiglu_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles,
                                                          const void *vec_a_mul, const void *vec_b_mul, int size_m, int size_k,
                                                          int size_n, int dtype, void *stream) {
+    forget_stale_error();
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
     if (size_n & 7) return QUEST_ERR_BAD_SHAPE;

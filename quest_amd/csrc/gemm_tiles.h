@@ -45,9 +45,10 @@ __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
 // no stream operation, nothing cached): the library keeps no state and a process may drive several devices.
 inline int device_cu_count(hipStream_t st) {
     int dev = 0, cus = 0;
-    if (hipStreamGetDevice(st, &dev) != hipSuccess && hipGetDevice(&dev) != hipSuccess) return 256;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
-    return cus;
+    const bool found = hipStreamGetDevice(st, &dev) == hipSuccess || hipGetDevice(&dev) == hipSuccess;
+    const bool counted = found && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0;
+    forget_stale_error();                      // a failed query must not be taken for the launch that follows
+    return counted ? cus : 256;
 }
 
 // gemm_big.hip: the large-tile kernel (K % 128 == 0, 4-byte aligned scale vectors); `duo` picks two workgroups of

@@ -93,6 +93,11 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
     const int lane = tid & 63;
     const int nchunks = K >> 3;
     const uint4 *xr = reinterpret_cast<const uint4 *>(x + (size_t)row * K);
+    // QUEST_QUANT_FROM_FP32: scale and codes come from the transform's fp32 output and the unrounded scale -- the
+    // arithmetic of the reference's evaluation-side fake quantiser (src/eval_hswag.py:201-214), which never holds the
+    // rotated tensor in 16 bits -- instead of from the dtype-rounded tensor the inference path materialises
+    const bool from_fp32 = (scale_rule & QUEST_QUANT_FROM_FP32) != 0;
+    scale_rule &= ~QUEST_QUANT_FROM_FP32;
 
     uint4 raw[NCHUNK];
 #pragma unroll
@@ -110,8 +115,8 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
             fwht128_chunk(y[i], lane);
 #pragma unroll
             for (int e = 0; e < 8; e++) y[i][e] *= had_scale;
-            raw[i] = pack8<DT>(y[i]);           // the transform's output exists only in dtype
-            unpack8<DT>(raw[i], y[i]);
+            raw[i] = pack8<DT>(y[i]);           // the transform's output exists only in dtype ...
+            if (!from_fp32) unpack8<DT>(raw[i], y[i]);     // ... unless the caller asks for the fp32 one to be quantised
         }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -130,16 +135,17 @@ hadamard_quantize_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ 
 
     // QUEST_SCALE_GAUSSIAN: the reference's rule from the row's mean square; QUEST_SCALE_ABSMAX: the row's largest
     // magnitude sits 7.5 steps out (a maximum is exact whatever the order, so this scale has no rounding slack)
-    uint32_t s16;
+    float s32;
     if (scale_rule == QUEST_SCALE_ABSMAX) {
         const float m = block_max_f<BLOCK>(amax, slots_f);
-        s16 = from_f32<DT>(__fadd_rn(__fdiv_rn(m, 7.5f), kScaleEps));
+        s32 = __fadd_rn(__fdiv_rn(m, 7.5f), kScaleEps);
     } else {
         const float total = block_sum_f<BLOCK>(sumsq, slots_f);
-        s16 = from_f32<DT>(scale_from_sumsq(total, K));
+        s32 = scale_from_sumsq(total, K);
     }
+    const uint32_t s16 = from_f32<DT>(s32);
     if (tid == 0) scale[row] = (uint16_t)s16;
-    const float s = to_f32<DT>(s16);
+    const float s = from_fp32 ? s32 : to_f32<DT>(s16);
 
     if (packed == nullptr && row_sum == nullptr) return;
     const float inv = quant_inv(s);
@@ -340,6 +346,7 @@ rope_kernel(uint16_t *__restrict__ x, const float *__restrict__ freqs, int n_row
 using namespace quest;
 
 extern "C" int quest_find_scale_int4(void *scale, const void *x, int group_size, int batch_size, int dtype, void *stream) {
+    forget_stale_error();
     if (!scale || !x) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (group_size <= 0 || batch_size <= 0 || (group_size & 7)) return QUEST_ERR_BAD_SHAPE;
@@ -355,6 +362,7 @@ extern "C" int quest_find_scale_int4(void *scale, const void *x, int group_size,
 extern "C" int quest_quantize_int4(void *x, const void *scale, int8_t *x_int, uint8_t *x_int_packed,
                                    int32_t *x_int_row_sum, int group_size, int batch_size, int do_dequantize,
                                    int dtype, void *stream) {
+    forget_stale_error();
     if (!x || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (group_size <= 0 || batch_size <= 0 || (group_size & 7)) return QUEST_ERR_BAD_SHAPE;
@@ -404,6 +412,7 @@ add_mul_vv_x8_kernel(uint16_t *__restrict__ d, const int32_t *__restrict__ a_add
 extern "C" int quest_add_mul_vv(void *mat_d, const int32_t *vec_a_add, const void *vec_a_mul, const int32_t *vec_b_add,
                                 const void *vec_b_mul, const int32_t *mat_c, int size_a, int size_b, int dtype,
                                 void *stream) {
+    forget_stale_error();
     if (!mat_d || !vec_a_add || !vec_a_mul || !vec_b_add || !vec_b_mul || !mat_c) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (size_a <= 0 || size_b <= 0) return QUEST_ERR_BAD_SHAPE;
@@ -433,6 +442,7 @@ extern "C" int quest_add_mul_vv(void *mat_d, const int32_t *vec_a_add, const voi
 
 extern "C" int quest_hadamard128(void *y, const void *x, int group_size, int batch_size, float had_scale, int dtype,
                                  void *stream) {
+    forget_stale_error();
     if (!y || !x) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
@@ -451,6 +461,7 @@ extern "C" int quest_hadamard128(void *y, const void *x, int group_size, int bat
 extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
                                             void *x_had, int group_size, int batch_size, float had_scale, int dtype,
                                             void *stream) {
+    forget_stale_error();
     if (!x || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     // the transform works on blocks of 128; without it (had_scale == 0) a row only has to be whole 16-byte chunks
@@ -471,10 +482,12 @@ extern "C" int quest_hadamard_quantize_int4(const void *x, void *scale, uint8_t 
 extern "C" int quest_hadamard_quantize_int4_rule(const void *x, void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
                                                  void *x_had, int group_size, int batch_size, float had_scale,
                                                  int scale_rule, int dtype, void *stream) {
+    forget_stale_error();
     if (scale_rule == QUEST_SCALE_GAUSSIAN)
         return quest_hadamard_quantize_int4(x, scale, x_int_packed, x_int_row_sum, x_had, group_size, batch_size, had_scale,
                                             dtype, stream);
-    if (scale_rule != QUEST_SCALE_ABSMAX) return QUEST_ERR_BAD_SHAPE;
+    if ((scale_rule & ~QUEST_QUANT_FROM_FP32) != QUEST_SCALE_ABSMAX && (scale_rule & ~QUEST_QUANT_FROM_FP32) != QUEST_SCALE_GAUSSIAN)
+        return QUEST_ERR_BAD_SHAPE;
     if (!x || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     // the transform works on blocks of 128; without it (had_scale == 0) a row only has to be whole 16-byte chunks
@@ -492,6 +505,7 @@ extern "C" int quest_rmsnorm_hadamard_quantize_int4(const void *x, const void *n
                                                     uint8_t *x_int_packed, int32_t *x_int_row_sum, void *x_had,
                                                     void *x_norm, int group_size, int batch_size, float had_scale,
                                                     int dtype, void *stream) {
+    forget_stale_error();
     if (!x || !norm_weight || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
@@ -505,6 +519,7 @@ extern "C" int quest_add_rmsnorm_hadamard_quantize_int4(void *x, const void *bra
                                                         void *scale, uint8_t *x_int_packed, int32_t *x_int_row_sum,
                                                         int group_size, int batch_size, float had_scale, int dtype,
                                                         void *stream) {
+    forget_stale_error();
     if (!x || !branch || !norm_weight || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
@@ -517,6 +532,7 @@ extern "C" int quest_add_rmsnorm_hadamard_quantize_int4(void *x, const void *bra
 extern "C" int quest_silu_mul_hadamard_quantize_int4(const void *gate_up, void *scale, uint8_t *x_int_packed,
                                                      int32_t *x_int_row_sum, void *x_had, void *x_act, int group_size,
                                                      int batch_size, float had_scale, int dtype, void *stream) {
+    forget_stale_error();
     if (!gate_up || !scale) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (group_size <= 0 || batch_size <= 0 || (group_size & 127)) return QUEST_ERR_BAD_SHAPE;
@@ -537,6 +553,7 @@ static int e2m3_rows_check(const void *x, const void *scale, const void *tiles, 
 extern "C" int quest_hadamard_quantize_e2m3(const void *x, void *scale, void *x_tiles, uint8_t *x_int_packed,
                                             int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size,
                                             float had_scale, int dtype, void *stream) {
+    forget_stale_error();
     const int rc = e2m3_rows_check(x, scale, x_tiles, group_size, batch_size, dtype);
     if (rc != QUEST_OK) return rc;
     if (!aligned(x_had, 16) || !aligned(x_int_packed, 4)) return QUEST_ERR_ALIGNMENT;
@@ -547,6 +564,7 @@ extern "C" int quest_hadamard_quantize_e2m3(const void *x, void *scale, void *x_
 extern "C" int quest_rmsnorm_hadamard_quantize_e2m3(const void *x, const void *norm_weight, float eps, void *scale,
                                                     void *x_tiles, void *x_norm, int group_size, int batch_size,
                                                     float had_scale, int dtype, void *stream) {
+    forget_stale_error();
     const int rc = e2m3_rows_check(x, scale, x_tiles, group_size, batch_size, dtype);
     if (rc != QUEST_OK) return rc;
     if (!norm_weight) return QUEST_ERR_NULL_POINTER;
@@ -558,6 +576,7 @@ extern "C" int quest_rmsnorm_hadamard_quantize_e2m3(const void *x, const void *n
 extern "C" int quest_add_rmsnorm_hadamard_quantize_e2m3(void *x, const void *branch, const void *norm_weight, float eps,
                                                         void *scale, void *x_tiles, int group_size, int batch_size,
                                                         float had_scale, int dtype, void *stream) {
+    forget_stale_error();
     const int rc = e2m3_rows_check(x, scale, x_tiles, group_size, batch_size, dtype);
     if (rc != QUEST_OK) return rc;
     if (!branch || !norm_weight) return QUEST_ERR_NULL_POINTER;
@@ -569,6 +588,7 @@ extern "C" int quest_add_rmsnorm_hadamard_quantize_e2m3(void *x, const void *bra
 extern "C" int quest_silu_mul_hadamard_quantize_e2m3(const void *gate_up, void *scale, void *x_tiles, void *x_act,
                                                      int group_size, int batch_size, float had_scale, int dtype,
                                                      void *stream) {
+    forget_stale_error();
     const int rc = e2m3_rows_check(gate_up, scale, x_tiles, group_size, batch_size, dtype);
     if (rc != QUEST_OK) return rc;
     if (!aligned(x_act, 16)) return QUEST_ERR_ALIGNMENT;
@@ -578,6 +598,7 @@ extern "C" int quest_silu_mul_hadamard_quantize_e2m3(const void *gate_up, void *
 
 extern "C" int quest_rope_interleaved(void *x, const float *freqs_cis, int n_rows, int seq_len, int row_stride,
                                       int rot_cols, int head_dim, int dtype, void *stream) {
+    forget_stale_error();
     if (!x || !freqs_cis) return QUEST_ERR_NULL_POINTER;
     if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
     if (n_rows <= 0 || seq_len <= 0 || rot_cols <= 0 || head_dim <= 0 || (head_dim & 7) || (rot_cols % head_dim) ||

@@ -30,7 +30,10 @@ def prefers_e2m3(m: int, k: int, n: int) -> bool:
     2048 to 13824 and M from 256 to 16384, the FP6 kernel wins from 66 tiles on (M = 1536 at N = 4096, M = 512 at
     N = 11008, M = 3072 at N = 2048) and loses below 64."""
     tiles = ((m + 255) // 256) * ((n + 255) // 256)
-    return MATRIX_PATH == 'fp6' and k % 128 == 0 and k <= 65536 and tiles >= E2M3_MIN_TILES and m * n < (1 << 31)
+    # K >= 2048: with shorter rows the GEMM is mostly epilogue either way, and what the FP6 kernel gains there (10-15 % on
+    # random codes) the activation kernels lose again writing tiles (scattered 16-byte pieces) instead of packed rows --
+    # measured on the 12-layer d = 1024 model: 6.17 ms per forward with tiles everywhere against 5.95 ms without
+    return (MATRIX_PATH == 'fp6' and k % 128 == 0 and 2048 <= k <= 65536 and tiles >= E2M3_MIN_TILES and m * n <= (1 << 30))
 
 
 def weight_tiles(w_int_packed: torch.Tensor) -> torch.Tensor:
@@ -101,7 +104,7 @@ def fused_matmul_dequantize_int4_bf16(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_
 
 
 def preprocess_weight(weight: torch.Tensor, use_sparse: bool = False, use_hadamard: bool = False, backend: str = 'hip',
-                      w_scale_mode: str = 'rms'):
+                      w_scale_mode: str = 'rms', quantize_from_fp32: bool = False):
     """utils.py:20-53, dense branch: (N, K) float weight -> (w_int_packed (N, K/2) uint8,
     w_scale (N, 1), w_add (N, 1) int32 = row sum of the codes + K/2, None)."""
     _check_backend(backend)
@@ -116,18 +119,20 @@ def preprocess_weight(weight: torch.Tensor, use_sparse: bool = False, use_hadama
     # (w_scale_mode: 'rms' is the reference's rule, 'absmax' puts the row's largest magnitude at the grid's edge)
     quest.hadamard_quantize_int4(weight, w_scale, w_int_packed, w_int_row_sum,
                                  hadamard_scale=WEIGHT_HADAMARD_SCALE if use_hadamard else 0.,
-                                 scale_rule={'rms': 'gaussian', 'absmax': 'absmax'}[w_scale_mode])
+                                 scale_rule={'rms': 'gaussian', 'absmax': 'absmax'}[w_scale_mode], from_fp32=quantize_from_fp32)
     w_add = w_int_row_sum + k // 2
     return w_int_packed, w_scale, w_add, None
 
 
 def linear_forward(activation, w_int_packed, w_scale, w_add, w_meta_e=None, out=None, _a_scale=None,
                    _a_int_packed=None, _a_int_row_sum=None, _c=None, use_hadamard=False, backend='hip', w_tiles=None,
-                   _a_tiles=None):
+                   _a_tiles=None, quantize_from_fp32=False):
     """utils.py:56-111, dense branch: out (M, N) = quantised activation @ quantised weight^T.
     Two launches: the fused Hadamard-scale-quantise-pack kernel, then the GEMM with the scale
     epilogue (the reference uses four).  With `w_tiles` (`weight_tiles(w_int_packed)`) and enough tokens the codes
-    travel as E2M3 tiles and the GEMM runs on the FP6 matrix instructions: the same output bits, faster."""
+    travel as E2M3 tiles and the GEMM runs on the FP6 matrix instructions: the same output bits, faster.
+    quantize_from_fp32 (with use_hadamard): the activation codes come from the fp32 transform (factor 2^-3.5, the
+    reference's evaluation-side arithmetic, src/eval_hswag.py:201-214) instead of from its 16-bit rounding."""
     _check_backend(backend)
     if w_meta_e is not None:
         raise NotImplementedError('4:8-sparse weights are not part of this build')
@@ -135,6 +140,11 @@ def linear_forward(activation, w_int_packed, w_scale, w_add, w_meta_e=None, out=
     dtype, device = activation.dtype, activation.device
     if out is None:
         out = torch.empty(m, n, dtype=dtype, device=device)
+    if quantize_from_fp32 and use_hadamard:
+        a_scale, a_int_packed, a_int_row_sum = quest.hadamard_quantize_int4(
+            activation, _a_scale, _a_int_packed, _a_int_row_sum, hadamard_scale=WEIGHT_HADAMARD_SCALE, from_fp32=True)
+        return quest.fused_matmul_dequantize_int4_int4t_bf16(mat_a=a_int_packed, mat_b=w_int_packed, vec_a_add=a_int_row_sum,
+                                                             vec_b_add=w_add, vec_a_mul=a_scale, vec_b_mul=w_scale, out=out)
     if w_tiles is not None and prefers_e2m3(m, k, n):
         a_scale, a_tiles = quest.hadamard_quantize_e2m3(activation, _a_scale, _a_tiles,
                                                         hadamard_scale=HADAMARD_ENTRY if use_hadamard else 0.)
@@ -169,10 +179,13 @@ class Linear4bit(nn.Module):
     def _configure(self, use_hadamard: bool, use_noop: bool) -> None:
         self.use_hadamard = use_hadamard
         self.use_noop = use_noop
+        # codes from the fp32 transform instead of its 16-bit rounding (see linear_forward); set before packing a weight
+        self.quantize_from_fp32 = getattr(self, 'quantize_from_fp32', False)
 
     def _install(self, weight: torch.Tensor, bias) -> None:
         """Pack `weight` (N, K) and keep `bias` (a tensor, a parameter or None) as a frozen parameter."""
-        packed, scale, add, _ = preprocess_weight(weight=weight, use_hadamard=self.use_hadamard)
+        packed, scale, add, _ = preprocess_weight(weight=weight, use_hadamard=self.use_hadamard,
+                                                  quantize_from_fp32=self.quantize_from_fp32)
         self._set_buffers(weight.shape, weight.dtype, packed, scale, add)
         if bias is None:
             self.bias = None
@@ -199,10 +212,12 @@ class Linear4bit(nn.Module):
         return self._tiles
 
     @classmethod
-    def from_weight(cls, weight: torch.Tensor, bias: torch.Tensor = None, use_hadamard: bool = False) -> 'Linear4bit':
+    def from_weight(cls, weight: torch.Tensor, bias: torch.Tensor = None, use_hadamard: bool = False,
+                    quantize_from_fp32: bool = False) -> 'Linear4bit':
         """Pack an existing (N, K) weight instead of a random one."""
         self = cls.__new__(cls)
         nn.Module.__init__(self)
+        self.quantize_from_fp32 = bool(quantize_from_fp32)
         self._configure(use_hadamard, False)
         self._install(weight, bias)
         return self
@@ -223,7 +238,10 @@ class Linear4bit(nn.Module):
 
     def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None) -> torch.Tensor:
         """The GEMM half of `linear_forward` on activations some fused producer kernel has already quantised:
-        (M, 1) scales, (M, K/2) codes, (M, 1) row sums -> (M, N)."""
+        (M, 1) scales, (M, K/2) codes, (M, 1) row sums -> (M, N).  In no-op mode the GEMM is skipped (zeros), which is
+        what prices the GEMMs of a producer-fused model: everything else, the quantising producers included, still runs."""
+        if self.use_noop:
+            return self._noop_output(a_scale)
         y = quest.fused_matmul_dequantize_int4_int4t_bf16(mat_a=a_int_packed, mat_b=self.w_int_packed,
                                                           vec_a_add=a_int_row_sum, vec_b_add=self.w_add,
                                                           vec_a_mul=a_scale, vec_b_mul=self.w_scale, out=out)
@@ -231,8 +249,16 @@ class Linear4bit(nn.Module):
             y += self.bias
         return y
 
+    def _noop_output(self, a_scale) -> torch.Tensor:
+        y = torch.zeros(a_scale.numel(), self.weight.size(0), dtype=a_scale.dtype, device=a_scale.device)
+        if self.bias is not None:
+            y += self.bias
+        return y
+
     def forward_tiles(self, a_scale, a_tiles, out=None) -> torch.Tensor:
         """The same for activations quantised to E2M3 tiles: the GEMM on the FP6 matrix instructions."""
+        if self.use_noop:
+            return self._noop_output(a_scale)
         y = quest.fused_matmul_dequantize_e2m3(a_tiles, self.w_tiles(), a_scale, self.w_scale, self.weight.size(1), out)
         if self.bias is not None:
             y += self.bias
@@ -250,7 +276,8 @@ class Linear4bit(nn.Module):
         else:
             m, k = rows.shape
             y = linear_forward(rows, self.w_int_packed, self.w_scale, self.w_add, self.w_meta_e,
-                               use_hadamard=self.use_hadamard, w_tiles=self.w_tiles() if prefers_e2m3(m, k, n) else None)
+                               use_hadamard=self.use_hadamard, quantize_from_fp32=self.quantize_from_fp32,
+                               w_tiles=self.w_tiles() if prefers_e2m3(m, k, n) and not self.quantize_from_fp32 else None)
         if self.bias is not None:
             y += self.bias
         return y.view(*lead, n)
@@ -284,7 +311,9 @@ def do_bench_network(f, M: int, K: int, N: int, dtype: torch.dtype, device: torc
     """utils.py:802-835: `f(activation_in (M, K), activation_out (M, N))` called `n_layers` times back to back on
     two views of one buffer (so that no call finds a fresh output allocation), timed as plain launches and as one
     replayed HIP graph; returns the smaller of the two, in seconds per layer."""
-    pool = torch.empty(M * max(K, N), dtype=dtype, device=device)
+    # Gaussian values, not the reference's uninitialised memory: the kernels' run time depends on the data (degenerate
+    # rows take a slower quantiser path, the clock follows the operands' power), and garbage would time something else
+    pool = torch.randn(M * max(K, N), dtype=torch.float32, device=device).to(dtype)
     a_in, a_out = pool[:M * K].view(M, K), pool[:M * N].view(M, N)
 
     def stack():

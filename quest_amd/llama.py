@@ -113,6 +113,8 @@ class LlamaMLP(nn.Module):
         """silu(w1 x) * w2 x, (M, hidden), from the codes of x; the gated unit runs in the GEMM's epilogue when that
         kernel takes the shape, otherwise in the torch expression on the plain GEMM's output."""
         m = a_int_packed.size(0)
+        if self.w12.use_noop:
+            return torch.zeros(m, self.c_proj.weight.size(1), dtype=a_scale.dtype, device=a_scale.device)
         if self.glu is not None and m > 64 and a_int_packed.size(1) % 64 == 0 and self.w12.bias is None:
             w_packed, w_scale, w_add = self.glu
             return quest.fused_matmul_dequantize_swiglu_int4_int4t(a_int_packed, w_packed, a_int_row_sum, w_add, a_scale, w_scale)
@@ -123,6 +125,8 @@ class LlamaMLP(nn.Module):
     def swiglu_tiles(self, a_scale, a_tiles):
         """The same from the E2M3 tiles of x, on the FP6 matrix instructions (needs enable_swiglu_epilogue())."""
         w_packed, w_scale, _ = self.glu
+        if self.w12.use_noop:
+            return torch.zeros(a_scale.numel(), self.c_proj.weight.size(1), dtype=a_scale.dtype, device=a_scale.device)
         if self.glu_tiles is None:
             self.glu_tiles = harness.weight_tiles(w_packed)
         return quest.fused_matmul_dequantize_e2m3(a_tiles, self.glu_tiles, a_scale, w_scale, w_packed.size(1) * 2, swiglu=True)
@@ -288,19 +292,24 @@ class Llama(nn.Module):
         return {'logits': logits}
 
 
-def _pack(linear: nn.Linear, use_hadamard: bool, use_noop: bool) -> harness.Linear4bit:
+def _pack(linear: nn.Linear, use_hadamard: bool, use_noop: bool, from_fp32: bool = False) -> harness.Linear4bit:
     m = harness.Linear4bit.from_weight(linear.weight.data, bias=None if linear.bias is None else linear.bias.data,
-                                       use_hadamard=use_hadamard)
+                                       use_hadamard=use_hadamard, quantize_from_fp32=from_fp32)
     m.use_noop = use_noop
     return m
 
 
 @torch.no_grad()
 def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, fuse_gate_up: bool = True,
-                   fuse_producers: bool = False, swiglu_epilogue: bool = True) -> Llama:
+                   fuse_producers: bool = False, swiglu_epilogue: bool = True, quantize_from_fp32: bool = False) -> Llama:
     """bench_e2e.py:77-97 on an existing model: every linear under `transformer` becomes a `Linear4bit` holding the
     packed INT4 form of that linear's own weight ('int4'), or the same module in no-op mode ('noop'); 'bf16' leaves
-    the dense linears.  The model must already sit on the GPU in bf16 or fp16."""
+    the dense linears.  The model must already sit on the GPU in bf16 or fp16.  quantize_from_fp32: weights and
+    activations are quantised from the fp32 transform, as the reference's evaluation-side fake quantiser does
+    (src/eval_hswag.py:201-214), not from its 16-bit rounding: the mode for checking a packed model against its
+    fake-quantised original (not available together with fuse_producers)."""
+    if quantize_from_fp32 and fuse_producers:
+        raise NotImplementedError('quantize_from_fp32 runs the unfused blocks: the producer-fused kernels quantise the 16-bit transform')
     if mode == 'bf16':
         for block in model.transformer.h:          # dense linears; only the rotary kernel replaces torch glue
             block.attn.fused_rope = bool(fuse_producers)
@@ -309,30 +318,42 @@ def quantize_model(model: Llama, mode: str = 'int4', use_hadamard: bool = True, 
         raise NotImplementedError(mode)
     noop = mode == 'noop'
     for block in model.transformer.h:
-        block.attn.c_attn = _pack(block.attn.c_attn, use_hadamard, noop)
-        block.attn.c_proj = _pack(block.attn.c_proj, use_hadamard, noop)
+        block.attn.c_attn = _pack(block.attn.c_attn, use_hadamard, noop, quantize_from_fp32)
+        block.attn.c_proj = _pack(block.attn.c_proj, use_hadamard, noop, quantize_from_fp32)
         mlp = block.mlp
         if fuse_gate_up:
             both = nn.Linear(mlp.w1.in_features, 2 * mlp.w1.out_features, bias=False, device=mlp.w1.weight.device,
                              dtype=mlp.w1.weight.dtype)
             both.weight.data = torch.cat([mlp.w1.weight.data, mlp.w2.weight.data], dim=0)
-            mlp.w12 = _pack(both, use_hadamard, noop)
+            mlp.w12 = _pack(both, use_hadamard, noop, quantize_from_fp32)
             mlp.w1 = mlp.w2 = None
         else:
-            mlp.w1 = _pack(mlp.w1, use_hadamard, noop)
-            mlp.w2 = _pack(mlp.w2, use_hadamard, noop)
-        mlp.c_proj = _pack(mlp.c_proj, use_hadamard, noop)
+            mlp.w1 = _pack(mlp.w1, use_hadamard, noop, quantize_from_fp32)
+            mlp.w2 = _pack(mlp.w2, use_hadamard, noop, quantize_from_fp32)
+        mlp.c_proj = _pack(mlp.c_proj, use_hadamard, noop, quantize_from_fp32)
         # the producer-fused kernels exist for the Hadamard variant, rows up to 32768 and the fused gate/up layout
-        block.attn.fused_rope = bool(fuse_producers and not noop)
-        block.fuse_producers = bool(fuse_producers and not noop and use_hadamard and fuse_gate_up and
+        # (in no-op mode the fused blocks keep their producers -- norms, residual additions, quantisers, rotary kernel --
+        # and only the GEMMs return zeros: the twin that prices the GEMMs of the producer-fused model)
+        block.attn.fused_rope = bool(fuse_producers)
+        block.fuse_producers = bool(fuse_producers and use_hadamard and fuse_gate_up and
                                     model.config.n_embd <= 32768 and model.config.hidden_dim <= 32768)
-        if fuse_producers and not noop and not block.fuse_producers:
+        if fuse_producers and not block.fuse_producers:
             import warnings
             warnings.warn('quantize_model: fuse_producers asked for, but this configuration (no Hadamard, separate gate / up '
                           'projections or rows over 32768) has no producer-fused kernels: the blocks run with torch glue')
         if block.fuse_producers and swiglu_epilogue and model.config.hidden_dim % 4 == 0:
             mlp.enable_swiglu_epilogue()
     return model
+
+
+def load_reference_checkpoint(model: Llama, path: str) -> Llama:
+    """Load a checkpoint file written by the reference's training loop (src/optim/utils.py:245-256: a dict with the
+    model's state dict under "model", next to optimizer, scheduler and iteration) into a dense model of this module.
+    The file is read with torch's weights-only loader, which unpickles tensors and plain containers and executes
+    nothing from the file; a bare state dict is accepted as well."""
+    ckpt = torch.load(path, map_location='cpu', weights_only=True)
+    state = ckpt['model'] if isinstance(ckpt, dict) and 'model' in ckpt and isinstance(ckpt['model'], dict) else ckpt
+    return load_reference_state_dict(model, state)
 
 
 @torch.no_grad()

@@ -162,6 +162,90 @@ def test_prefill_gemm_full_size(quest, shape):
     assert rel <= 1e-2, rel
 
 
+@pytest.mark.parametrize('shape', [(4096, 4096, 11008), (16384, 1024, 3072), (16384, 2816, 1024), (9000, 512, 4104)])
+def test_prefill_gemm_e2m3_full_size(quest, shape):
+    """The FP6 kernel at the same sizes, by the same method: its output is the epilogue formula on the exact integer
+    matrix -- 2 C + a_add + b_add recovered from checksums and sampled rows as above -- everywhere, bit for bit."""
+    m, k, n = shape
+    a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=0)
+    gap, gbp = ap.to(DEV), bp.to(DEV)
+    g_a_add, g_b_add, g_a_mul, g_b_mul = (t.to(DEV) for t in (a_add, b_add, a_mul, b_mul))
+    d = quest.fused_matmul_dequantize_e2m3(quest.int4_to_e2m3_tiles(gap), quest.int4_to_e2m3_tiles(gbp), g_a_mul, g_b_mul, k)
+    # exact integers on the GPU in fp64 (|values| < 2^53), independent of either GEMM kernel
+    ga, gb = a.to(DEV).double(), b.to(DEV).double()
+    gen = torch.Generator().manual_seed(2)
+    rows = torch.randperm(m, generator=gen)[:64].to(DEV)
+    c_rows = (ga[rows] @ gb.T).to(torch.int32)
+    lhs = (c_rows * 2 + g_a_add[rows] + g_b_add.T).float()
+    rhs = (0.5 * g_a_mul[rows].float()) * g_b_mul.float().T
+    assert torch.equal(bits(d[rows]), bits((lhs * rhs).to(d.dtype)))
+    # everywhere: against the INT8 kernel, whose int32 matrix the test above pins by checksums
+    want = quest.fused_matmul_dequantize_int4_int4t_bf16(gap, gbp, g_a_add, g_b_add, g_a_mul, g_b_mul)
+    assert torch.equal(bits(d), bits(want))
+
+
+def test_swiglu_gemm_full_size(quest):
+    """The gate/up GEMM of Llama-7B with the gated unit in its epilogue, M = 4096, K = 4096, 2 H = 22016: equal to the
+    plain fused GEMM (pinned above) on the same rows followed by torch's silu(gate) * up -- within 2 ulp on under 2 % of
+    the elements (the fast exponential) everywhere against torch on the GPU and on 64 sampled rows against torch on the
+    CPU; the INT8 and the FP6 kernel agree bit for bit."""
+    m, k, n = 4096, 4096, 22016
+    h = n // 2
+    a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=5, dtype=torch.bfloat16)
+    gap, gbp = ap.to(DEV), bp.to(DEV)
+    g_a_add, g_b_add, g_a_mul, g_b_mul = (t.to(DEV) for t in (a_add, b_add, a_mul * 0.1, b_mul * 0.1))
+    p = quest.swiglu_interleave_rows(h, device=DEV)
+    bpi, bai, bmi = gbp[p].contiguous(), g_b_add[p].contiguous(), g_b_mul[p].contiguous()
+    got = quest.fused_matmul_dequantize_swiglu_int4_int4t(gap, bpi, g_a_add, bai, g_a_mul, bmi)
+    assert got.shape == (m, h)
+    got6 = quest.fused_matmul_dequantize_e2m3(quest.int4_to_e2m3_tiles(gap), quest.int4_to_e2m3_tiles(bpi), g_a_mul, bmi, k, swiglu=True)
+    assert torch.equal(bits(got), bits(got6))
+    gate_up = quest.fused_matmul_dequantize_int4_int4t_bf16(gap, gbp, g_a_add, g_b_add, g_a_mul, g_b_mul)     # (M, 2 H): gates, then ups
+    want = torch.nn.functional.silu(gate_up[:, :h].float()).to(gate_up.dtype).float() * gate_up[:, h:].float()
+    want = want.to(gate_up.dtype)
+    d = (bits(got) - bits(want)).abs()
+    assert int(d.max()) <= 2 and float((d != 0).float().mean()) < 0.02, (int(d.max()), float((d != 0).float().mean()))
+    gen = torch.Generator().manual_seed(6)
+    rows = torch.randperm(m, generator=gen)[:64]
+    cpu = gate_up[rows.to(DEV)].cpu()
+    want_cpu = torch.nn.functional.silu(cpu[:, :h]) * cpu[:, h:]
+    dc = (bits(got[rows.to(DEV)].cpu()) - bits(want_cpu)).abs()
+    assert int(dc.max()) <= 2 and float((dc != 0).float().mean()) < 0.02
+
+
+@pytest.mark.parametrize('m', [1, 8, 16])
+@pytest.mark.parametrize('kn', [(4096, 4096), (11008, 4096)])
+def test_decode_layer_as_one_workload(quest, m, kn, capsys):
+    """The decode configuration as the layer it is: fp16 randn activations -> fused Hadamard-quantise -> weight-streaming
+    GEMM, through harness.linear_forward.  The output equals the oracle's GEMM + epilogue on the codes the kernel produced,
+    bit for bit; those codes against the full oracle pipeline on the same x (F.linear Hadamard, torch-CPU scale,
+    quantiser) are counted and bounded."""
+    from quest_amd import harness
+    k, n = kn
+    g = torch.Generator().manual_seed(100 + m)
+    x = torch.randn(m, k, generator=g).half()
+    b = torch.randint(-8, 8, (n, k), generator=g, dtype=torch.int8)
+    w_packed = qo.pack_int4(b)
+    w_scale = (torch.rand(n, 1, generator=g) * 0.09 + 0.01).half()
+    w_add = (b.to(torch.int32).sum(-1, keepdim=True) + k // 2).to(torch.int32)
+    a_scale = torch.empty(m, 1, dtype=torch.float16, device=DEV)
+    a_packed = torch.empty(m, k // 2, dtype=torch.uint8, device=DEV)
+    a_row_sum = torch.empty(m, 1, dtype=torch.int32, device=DEV)
+    y = harness.linear_forward(x.to(DEV), w_packed.to(DEV), w_scale.to(DEV), w_add.to(DEV), use_hadamard=True,
+                               _a_scale=a_scale, _a_int_packed=a_packed, _a_int_row_sum=a_row_sum)
+    want = qo.fused_matmul_dequantize_int4_int4t(a_packed.cpu(), w_packed, a_row_sum.cpu(), w_add, a_scale.cpu(), w_scale, via='fp32')
+    assert torch.equal(bits(y.cpu()), bits(want))
+    _, o_scale, o_packed, _ = qo.hadamard_quantize_int4(x, hadamard='matmul')
+    differ = float((qo.unpack_int4(a_packed.cpu()) != qo.unpack_int4(o_packed)).float().mean())
+    scale_ulps = int((bits(a_scale.cpu()) - bits(o_scale)).abs().max())
+    with capsys.disabled():
+        print(f'\n[decode layer M={m} K={k} N={n}] activation codes differing from the oracle pipeline: {100 * differ:.3f} %, '
+              f'scale within {scale_ulps} ulp')
+    assert differ < 0.02 and scale_ulps <= 1
+    ref = qo.linear_forward(x, w_packed, w_scale, w_add, use_hadamard=True, hadamard='matmul', via='fp32').double()
+    assert float((y.cpu().double() - ref).norm() / ref.norm()) < 1e-2
+
+
 @pytest.mark.parametrize('m', [1, 8, 16])
 @pytest.mark.parametrize('kn', [(4096, 4096), (11008, 4096), (4096, 11008)])
 def test_decode_gemm_full_shapes(quest, m, kn):
@@ -173,6 +257,60 @@ def test_decode_gemm_full_shapes(quest, m, kn):
     d = quest.fused_matmul_dequantize_int4_int4t_bf16(ap.to(DEV), bp.to(DEV), a_add.to(DEV), b_add.to(DEV), a_mul.to(DEV), b_mul.to(DEV))
     want_d = qo.add_mul_vv(a_add, a_mul, b_add, b_mul, want_c)
     assert torch.equal(bits(d.cpu()), bits(want_d))
+
+
+@pytest.mark.parametrize('m', [1, 5, 16])
+@pytest.mark.parametrize('kn', [(4096, 4096), (11008, 4096), (4096, 11008), (1024, 3072), (4096, 4090), (32768, 1000)])
+def test_decode_gemm_split_k(quest, m, kn):
+    """K split across workgroups through a caller-owned workspace: bit-exact against the oracle, the same workspace
+    reused across shapes and calls without clearing it (every call leaves its counters at zero), also from a HIP graph."""
+    k, n = kn
+    a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=11 + m)
+    want_d = qo.add_mul_vv(a_add, a_mul, b_add, b_mul, (a.double() @ b.double().T).to(torch.int32))
+    if 'work' not in _SPLIT_K_STATE:
+        _SPLIT_K_STATE['work'] = quest.gemm_workspace(DEV)
+    work = _SPLIT_K_STATE['work']
+    assert quest.gemm_workspace_bytes(m, k, n) <= work.numel()
+    args = [t.to(DEV) for t in (ap, bp, a_add, b_add, a_mul, b_mul)]
+    for _ in range(3):
+        d = quest.fused_matmul_dequantize_int4_int4t_bf16(*args, workspace=work)
+        assert torch.equal(bits(d.cpu()), bits(want_d))
+    assert int(work[:16384].view(torch.int32).abs().max()) == 0
+    out = torch.empty_like(d)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        quest.fused_matmul_dequantize_int4_int4t_bf16(*args, out=out, workspace=work)
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        quest.fused_matmul_dequantize_int4_int4t_bf16(*args, out=out, workspace=work)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(bits(out.cpu()), bits(want_d))
+
+
+_SPLIT_K_STATE = {}
+
+
+def test_decode_gemm_split_k_falls_back(quest):
+    """No workspace, one too small, or a shape that does not split: the plain kernel runs, same result."""
+    m, k, n = 4, 4096, 4096
+    a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=2)
+    args = [t.to(DEV) for t in (ap, bp, a_add, b_add, a_mul, b_mul)]
+    want = quest.fused_matmul_dequantize_int4_int4t_bf16(*args)
+    small = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    assert quest.gemm_workspace_bytes(m, k, n) > small.numel()
+    assert torch.equal(bits(quest.fused_matmul_dequantize_int4_int4t_bf16(*args, workspace=small)), bits(want))
+    assert quest.gemm_workspace_bytes(64, k, n) == 0 and quest.gemm_workspace_bytes(4, 4160, n) == 0
+    m = 64
+    a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=3)
+    args = [t.to(DEV) for t in (ap, bp, a_add, b_add, a_mul, b_mul)]
+    work = quest.gemm_workspace(DEV)
+    assert torch.equal(bits(quest.fused_matmul_dequantize_int4_int4t_bf16(*args, workspace=work)),
+                       bits(quest.fused_matmul_dequantize_int4_int4t_bf16(*args)))
 
 
 def test_forward_full_config():

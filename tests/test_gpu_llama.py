@@ -190,3 +190,17 @@ def test_trained_checkpoint_path_against_fake_quant_model(llama, dtype, capsys):
         print(f'\n[trained-checkpoint path, {dtype}] packed GPU logits vs fake-quant model: {err:.3f}; CPU oracle of the '
               f'inference path vs fake-quant model: {err_ref:.3f}; fake-quant vs dense model: {gap:.3f}')
     assert err < 0.25 and err < 1.5 * err_ref + 0.02 and err < gap, (err, err_ref, gap)
+    # the same checkpoint packed and run with the codes taken from the fp32 transform, as the fake quantiser takes them:
+    # the per-layer distance falls under 1e-2 (tests/test_gpu_parity.py) and the model-level one with it
+    torch.manual_seed(12)
+    model32 = llama.Llama(cfg).to(dtype).to(DEV).eval()
+    llama.load_reference_state_dict(model32, ckpt)
+    llama.quantize_model(model32, 'int4', use_hadamard=True, fuse_gate_up=True, quantize_from_fp32=True)
+    with torch.no_grad():
+        got32 = model32(ids.to(DEV), all_logits=True)['logits'].double().cpu()
+    err32 = float((got32 - fake).norm() / fake.norm())
+    with capsys.disabled():
+        print(f'[trained-checkpoint path, {dtype}] quantised from the fp32 transform: {err32:.3f} from the fake-quant model')
+    # (random weights amplify every flipped code, and torch's GPU and CPU glue round bf16 differently between the two
+    # forwards, so the model-level distance stays far above the per-layer one)
+    assert err32 < err, (err32, err)

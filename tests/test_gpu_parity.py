@@ -397,6 +397,32 @@ def test_packed_linear_against_training_side_fake_quant(quest, dtype):
     assert err < 1.25 * err_ref + 1e-3, (float(err), float(err_ref))
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_packed_linear_quantised_from_fp32_meets_the_fake_quant_bar(quest, dtype, capsys):
+    """With `quantize_from_fp32` weights and activations are quantised from the fp32 transform (factor 2^-3.5) and the
+    unrounded scale -- the arithmetic of the evaluation-side fake quantiser (src/eval_hswag.py:201-214) -- and the packed
+    layer agrees with the fake-quantised one to <= 1e-2 relative; what is left is the 16-bit rounding of the stored
+    scales and of the output."""
+    from quest_amd import harness
+    g = torch.Generator().manual_seed(40)
+    x = torch.randn(192, 1024, generator=g).to(dtype)
+    w = (torch.randn(320, 1024, generator=g) * 0.02).to(dtype)
+    want = qo.fake_quant_linear(x, w).double()
+    layer = harness.Linear4bit.from_weight(w.to(DEV), use_hadamard=True, quantize_from_fp32=True)
+    got = layer(x.to(DEV)).double().cpu()
+    plain = harness.Linear4bit.from_weight(w.to(DEV), use_hadamard=True)(x.to(DEV)).double().cpu()
+    err = float((got - want).norm() / want.norm())
+    err_plain = float((plain - want).norm() / want.norm())
+    # the codes themselves: the fake quantiser's levels 0..15 are the codes + 8
+    wq, _, _ = qo.fake_quant_hadamard(w)
+    codes = qo.unpack_int4(layer.w_int_packed.cpu()).to(torch.float32) + 8
+    differ = float((codes != wq).float().mean())
+    with capsys.disabled():
+        print(f'\n[fake-quant bar, {dtype}] from fp32: {err:.2e} (weight codes differing {differ:.2e}); default path: {err_plain:.2e}')
+    assert err <= 1e-2, err
+    assert differ < 1e-3, differ
+
+
 # --------------------------------------------------------------------------- producers fused in front
 def _ulp_stats(got, want):
     d = ulp_diff(got, want)

@@ -16,6 +16,8 @@ import random
 import pytest
 import torch
 
+from oracle import quest_oracle as qo
+
 pytestmark = pytest.mark.gpu
 DEV = 'cuda:0'
 
@@ -80,6 +82,12 @@ def test_gemm_random_shapes(quest, seed):
         lhs = (want_c * 2 + a_add + b_add.T).float()
         rhs = (0.5 * a_mul.float()) * b_mul.float().T
         assert torch.equal(bits(got_d), bits((lhs * rhs).to(dtype))), (m, k, n, dtype)
+        if k % 128 == 0:
+            # the FP6 kernel on the same codes as E2M3 tiles: the add vectors are the codes' own sums there
+            ua, ub = unpack(a).to(torch.int32), unpack(b).to(torch.int32)
+            lhs6 = (want_c * 2 + ua.sum(-1, keepdim=True) + (ub.sum(-1, keepdim=True) + k // 2).T).float()
+            got6 = quest.fused_matmul_dequantize_e2m3(quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(b), a_mul, b_mul, k)
+            assert torch.equal(bits(got6), bits((lhs6 * rhs).to(dtype))), (m, k, n, dtype)
 
 
 @pytest.mark.parametrize('seed', [201, 202])
@@ -91,7 +99,14 @@ def test_activation_kernel_random_shapes(quest, seed):
         k = 128 * rng.choice([1, 2, 3, 4, 5, 8, 11, 16, 22, 32, 33, 40, 64, 86, 128, 200, 256])
         m = min(m, max(1, int(2.0e7 // k)))
         dtype = rng.choice([torch.bfloat16, torch.float16])
-        x = (torch.randn(m, k, device=DEV, generator=g) * (torch.rand(m, 1, device=DEV, generator=g) * 4 + 0.05)).to(dtype)
+        xf = torch.randn(m, k, device=DEV, generator=g) * (torch.rand(m, 1, device=DEV, generator=g) * 4 + 0.05)
+        # rows of small and large magnitude, and one whose values and scale lie in the dtype's subnormals (fp16: below
+        # 6.1e-5; the scale stays above zero -- what a zero scale gives is fixed by tests/test_gpu_configs.py)
+        if m >= 4:
+            xf[0] *= 1e-3
+            xf[1] *= 1e3
+            xf[2] *= 2e-6 if dtype == torch.float16 else 1e-30
+        x = xf.to(dtype)
         x_had = torch.empty_like(x)
         scale, packed, row_sum = quest.hadamard_quantize_int4(x, x_had=x_had)
         s2 = quest.find_scale_int4(x_had)
@@ -99,7 +114,18 @@ def test_activation_kernel_random_shapes(quest, seed):
         _, _, p2, r2 = quest.quantize_int4(x_had.clone(), scale, x_int_packed=torch.empty_like(packed),
                                            x_int_row_sum=torch.empty_like(row_sum))
         assert torch.equal(packed, p2) and torch.equal(row_sum, r2), (m, k, dtype)
-        if k > 4096:
+        # the two kernels share their quantiser helpers, so a sample of rows also goes through the CPU oracle
+        # (IEEE divide, floor, clamp: gemm-quest/benchmarks/utils.py:334-365) with the kernel's transform and scale
+        sample = list(range(min(m, 6)))
+        o_packed = torch.empty(len(sample), k // 2, dtype=torch.uint8)
+        o_sum = torch.empty(len(sample), 1, dtype=torch.int32)
+        qo.quantize_int4(x_had[sample].cpu().clone(), scale[sample].cpu(), None, o_packed, o_sum, False)
+        assert torch.equal(packed[sample].cpu(), o_packed) and torch.equal(row_sum[sample].cpu(), o_sum), (m, k, dtype)
+        # ... and the E2M3 tiles hold the same codes
+        _, tiles = quest.hadamard_quantize_e2m3(x)
+        assert torch.equal(quest.int4_to_e2m3_tiles(packed).view(-1, 1536)[: (m // 32) * (k // 64)],
+                           tiles.view(-1, 1536)[: (m // 32) * (k // 64)]), (m, k, dtype)
+        if k > 4096 and rng.random() < 0.5:
             continue
         w = (1 + 0.1 * torch.randn(k, device=DEV, generator=g)).to(dtype)
         x_norm = torch.empty_like(x)

@@ -145,3 +145,25 @@ def test_reference_checkpoint_names_load():
     del sd['_orig_mod.module.lm_head.weight']
     with pytest.raises(KeyError):
         llama.load_reference_state_dict(model, sd)
+
+
+def test_reference_checkpoint_file_loads_weights_only(tmp_path):
+    """A file as the reference's training loop writes it (src/optim/utils.py:245-256: model / optimizer / scheduler /
+    itr, parameter names behind the training wrapper's prefix), read back with the weights-only loader."""
+    torch.manual_seed(3)
+    cfg = llama.LlamaConfig(n_layer=1, n_embd=128, n_head=2, vocab_size=64, sequence_length=16)
+    donor = llama.Llama(cfg)
+    state = {'_orig_mod.module.' + k: v.detach().clone() for k, v in donor.state_dict().items()}
+    path = tmp_path / 'main.pt'
+    torch.save({'model': state, 'optimizer': {'state': {}, 'param_groups': [{'lr': 1e-3}]}, 'scheduler': {'last_epoch': 7}, 'itr': 7}, path)
+    torch.manual_seed(4)
+    model = llama.Llama(cfg)
+    llama.load_reference_checkpoint(model, str(path))
+    for k, v in donor.state_dict().items():
+        assert torch.equal(model.state_dict()[k], v), k
+    # a bare state dict is accepted too
+    torch.save(state, tmp_path / 'bare.pt')
+    torch.manual_seed(5)
+    other = llama.Llama(cfg)
+    llama.load_reference_checkpoint(other, str(tmp_path / 'bare.pt'))
+    assert torch.equal(other.lm_head.weight, donor.lm_head.weight)
