@@ -179,6 +179,7 @@ gemm_w4a4_decode_kernel(void *__restrict__ out, const uint8_t *__restrict__ act,
 // per wave for long rows.  Workspace: ceil(N / 16) counters (zero before the first use, zero again after every launch),
 // then, from byte kSplitPartialsAt on, ceil(N / 16) x S tiles of 256 ints.
 constexpr int kSplitWaves = 4;
+constexpr int kMaxSplits = 8;
 constexpr size_t kSplitPartialsAt = 16384;          // room for 4096 counters: N <= 65536
 
 template <int OUT>
@@ -247,21 +248,28 @@ gemm_w4a4_decode_splitk_kernel(void *__restrict__ out, const uint8_t *__restrict
         for (int e = 0; e < 4; e++) sum[e] += p[e];
     }
     if (splits > 1) {
-        // publish, count, and let the last arriver gather.  The fences are device-wide releases / acquires: the slices of
-        // one channel tile may run on different XCDs, whose L2 caches do not see each other's lines otherwise.
-        int *mine = partials + ((size_t)tile * splits + blockIdx.y) * 256;
-        *reinterpret_cast<v4i *>(mine + lane * 4) = sum;
-        __threadfence();
+        // Publish, count, and let the last arriver gather.  The slices of one channel tile may run on different XCDs, whose
+        // L2 caches do not see each other's lines; a device-wide release / acquire fence would write back and invalidate a
+        // whole L2 per workgroup (measured: ten times the kernel's time).  Instead the partial tiles travel past the
+        // caches: stores and loads with both coherence bits set go to the memory side, the counter is a device-scope
+        // atomic, and the store is complete (vmcnt) before the count.
+        const __amdgpu_buffer_rsrc_t pr = __builtin_amdgcn_make_buffer_rsrc((void *)partials, 0, (int)(gridDim.x * splits * 1024), 0x00020000);
+        constexpr int kPastCaches = 1 | 16;             // sc0 sc1
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int, sum), pr, (int)((tile * splits + blockIdx.y) * 1024 + lane * 16), 0, kPastCaches);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         int arrived = 0;
-        if (lane == 0) arrived = __hip_atomic_fetch_add(counters + tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__builtin_amdgcn_readfirstlane(arrived) != splits - 1) return;
-        __threadfence();
-        sum = v4i{0, 0, 0, 0};
-        for (int sl = 0; sl < splits; sl++) {
-            const v4i p = *reinterpret_cast<const v4i *>(partials + ((size_t)tile * splits + sl) * 256 + lane * 4);
+        asm volatile("" ::: "memory");
+        v4i part[kMaxSplits];                          // every slice's tile in flight at once; slices past the last read as zero
 #pragma unroll
-            for (int e = 0; e < 4; e++) sum[e] += p[e];
-        }
+        for (int sl = 0; sl < kMaxSplits; sl++)
+            part[sl] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(pr, sl < splits ? (int)((tile * splits + sl) * 1024 + lane * 16) : (int)0x80000000, 0, kPastCaches));
+        sum = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int sl = 0; sl < kMaxSplits; sl++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) sum[e] += part[sl][e];
         if (lane == 0) __hip_atomic_store(counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     // ready for the next launch
     }
 
@@ -320,13 +328,17 @@ static int launch_out(void *out, const uint8_t *a, const uint8_t *b, const int32
     return launch_status();
 }
 
-// How many slices of K pay for M <= 16 tokens: enough workgroups to fill the chip several times over, at least two
-// 256-k chunks per wave of a slice.
+// How many slices of K pay for M <= 16 tokens.  The hand-off through memory (store past the caches, count, load) costs
+// 2-2.5 us, more than the whole kernel above takes on an 8 MB layer, so slices pay only where that kernel's few
+// workgroups each walk a long row: measured wins (6.9-12.3 us against 11.2-16.7 us) for K >= 32768 with N <= 2048 and
+// K >= 16384 with N <= 1024, losses of 1.5-4 us everywhere else, the Llama decode layers included.  Then: enough
+// workgroups to fill the chip several times over, at least two 256-k chunks per wave of a slice.
 static int decode_splits(int K, int N) {
     const int tiles = (N + kChannels - 1) / kChannels;
     const int n_chunks = ((K >> 1) + kChunkB - 1) / kChunkB;
+    if (!(n_chunks >= 128 && tiles <= 128) && !(n_chunks >= 64 && tiles <= 64)) return 1;
     int s = 1;
-    while (s < 8 && tiles * s * 2 <= 2048 && n_chunks / (s * 2) >= kSplitWaves) s *= 2;
+    while (s < kMaxSplits && tiles * s * 2 <= 2048 && n_chunks / (s * 2) >= kSplitWaves) s *= 2;
     return s;
 }
 

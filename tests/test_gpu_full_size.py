@@ -260,10 +260,11 @@ def test_decode_gemm_full_shapes(quest, m, kn):
 
 
 @pytest.mark.parametrize('m', [1, 5, 16])
-@pytest.mark.parametrize('kn', [(4096, 4096), (11008, 4096), (4096, 11008), (1024, 3072), (4096, 4090), (32768, 1000)])
+@pytest.mark.parametrize('kn', [(32768, 512), (32768, 1000), (32768, 2048), (16384, 1024), (65536, 250), (16384, 1022), (4096, 4096), (11008, 4096)])
 def test_decode_gemm_split_k(quest, m, kn):
-    """K split across workgroups through a caller-owned workspace: bit-exact against the oracle, the same workspace
-    reused across shapes and calls without clearing it (every call leaves its counters at zero), also from a HIP graph."""
+    """K split across workgroups through a caller-owned workspace (long rows, few channels; the last two shapes do not
+    split and take the plain kernel): bit-exact against the oracle, the same workspace reused across shapes and calls
+    without clearing it (every call leaves its counters at zero), also from a HIP graph."""
     k, n = kn
     a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=11 + m)
     want_d = qo.add_mul_vv(a_add, a_mul, b_add, b_mul, (a.double() @ b.double().T).to(torch.int32))
@@ -271,6 +272,7 @@ def test_decode_gemm_split_k(quest, m, kn):
         _SPLIT_K_STATE['work'] = quest.gemm_workspace(DEV)
     work = _SPLIT_K_STATE['work']
     assert quest.gemm_workspace_bytes(m, k, n) <= work.numel()
+    assert (quest.gemm_workspace_bytes(m, k, n) > 0) == (k >= 16384)
     args = [t.to(DEV) for t in (ap, bp, a_add, b_add, a_mul, b_mul)]
     for _ in range(3):
         d = quest.fused_matmul_dequantize_int4_int4t_bf16(*args, workspace=work)
@@ -297,14 +299,15 @@ _SPLIT_K_STATE = {}
 
 def test_decode_gemm_split_k_falls_back(quest):
     """No workspace, one too small, or a shape that does not split: the plain kernel runs, same result."""
-    m, k, n = 4, 4096, 4096
+    m, k, n = 4, 32768, 512
     a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=2)
     args = [t.to(DEV) for t in (ap, bp, a_add, b_add, a_mul, b_mul)]
     want = quest.fused_matmul_dequantize_int4_int4t_bf16(*args)
     small = torch.zeros(4096, dtype=torch.uint8, device=DEV)
     assert quest.gemm_workspace_bytes(m, k, n) > small.numel()
     assert torch.equal(bits(quest.fused_matmul_dequantize_int4_int4t_bf16(*args, workspace=small)), bits(want))
-    assert quest.gemm_workspace_bytes(64, k, n) == 0 and quest.gemm_workspace_bytes(4, 4160, n) == 0
+    assert quest.gemm_workspace_bytes(64, k, n) == 0 and quest.gemm_workspace_bytes(4, 32768 + 64, n) == 0
+    assert quest.gemm_workspace_bytes(4, 4096, 4096) == 0
     m = 64
     a, b, ap, bp, a_add, b_add, a_mul, b_mul = _gemm_inputs(m, k, n, seed=3)
     args = [t.to(DEV) for t in (ap, bp, a_add, b_add, a_mul, b_mul)]
