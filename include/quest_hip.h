@@ -108,6 +108,22 @@ int quest_fused_matmul_dequantize_int4_int4t_ws(void *mat_d, const uint8_t *mat_
                                                 void *stream);
 
 /*
+ * quest_fused_matmul_dequantize_int4_int4t_ws for callers that cannot allocate a workspace (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  The workspace is an
+ * array inside the library, quest_gemm_noalloc_scratch_bytes() bytes (1,064,960) on every GPU the library runs on,
+ * held until the process ends; the call allocates and frees nothing.  size_m <= 16 (QUEST_ERR_UNSUPPORTED above, or
+ * if a shape ever needed more than the array holds); shapes that do not split K run the plain kernel.  Same outputs
+ * bit for bit.  Every call on one GPU shares that GPU's array: calls that may overlap in time on one GPU (different
+ * streams, different threads) race -- give those quest_fused_matmul_dequantize_int4_int4t_ws and a workspace each.
+ * The first call on a device looks the array up (hipGetSymbolAddress); make it before capturing a graph.
+ */
+size_t quest_gemm_noalloc_scratch_bytes(void);
+int quest_fused_matmul_dequantize_int4_int4t_noalloc(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                     const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                     const void *vec_a_mul, const void *vec_b_mul, int size_m, int size_k,
+                                                     int size_n, int dtype, void *stream);
+
+/*
  * y = block-128 Walsh-Hadamard transform of every row of x along K, fp32 butterflies, * had_scale,
  * one rounding to dtype.  had_scale = 181/2048 reproduces F.linear(x.view(-1,128), HADAMARD_MATRIX)
  * (benchmarks/utils.py:17,89-90: the matrix entries are bf16(2^-3.5) = 181/2048); had_scale = 2^-3.5

@@ -38,6 +38,8 @@ SIGNATURES = {
     'quest_silu_mul_hadamard_quantize_int4': [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     'quest_gemm_workspace_bytes': [_i, _i, _i],
     'quest_fused_matmul_dequantize_int4_int4t_ws': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp],
+    'quest_gemm_noalloc_scratch_bytes': [],
+    'quest_fused_matmul_dequantize_int4_int4t_noalloc': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     'quest_e2m3_tiles_bytes': [_i, _i],
     'quest_int4_to_e2m3_tiles': [_vp, _vp, _i, _i, _vp],
     'quest_fused_matmul_dequantize_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
@@ -50,7 +52,7 @@ SIGNATURES = {
 }
 # entry points that do not return an int status
 _RESTYPES = {'quest_status_string': ctypes.c_char_p, 'quest_e2m3_tiles_bytes': ctypes.c_size_t,
-             'quest_gemm_workspace_bytes': ctypes.c_size_t}
+             'quest_gemm_workspace_bytes': ctypes.c_size_t, 'quest_gemm_noalloc_scratch_bytes': ctypes.c_size_t}
 
 _lib = None
 

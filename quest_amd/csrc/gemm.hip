@@ -19,6 +19,8 @@
 //                                               staged through registers into int8 LDS tiles.
 #include "gemm_tiles.h"
 
+#include <mutex>
+
 namespace quest {
 
 static int gemm_check(const void *out, const uint8_t *a, const uint8_t *b, int M, int K, int N) {
@@ -137,6 +139,61 @@ extern "C" int quest_fused_matmul_dequantize_int4_int4t_ws(void *mat_d, const ui
     const int out_kind = dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16;
     const int split = launch_gemm_decode_splitk(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m,
                                                 size_k, size_n, workspace, workspace_bytes, (hipStream_t)stream);
+    if (split != QUEST_ERR_UNSUPPORTED) return split;
+    return gemm_launch(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m, size_k, size_n,
+                       (hipStream_t)stream);
+}
+
+// ---- the same GEMM for callers that cannot allocate ------------------------------------------------------------------
+// The split-K workspace lives in the library: one array per GPU (every device that loads this code object holds its own
+// copy at its own address, zero at load, until the process ends).  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and every other use of the memory take the address that call returns.
+namespace {
+constexpr size_t kScratchBytes = 16384 + (1u << 20);      // counters + 1024 partial tiles: the most any shape that splits uses
+constexpr int kScratchDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+void *scratch_of_device[kScratchDevices];
+std::mutex scratch_mutex;
+
+int scratch_here(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchDevices) {
+        (void)hipGetLastError();
+        return QUEST_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> hold(scratch_mutex);
+    if (scratch_of_device[dev] == nullptr) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return QUEST_ERR_LAUNCH;
+        }
+        scratch_of_device[dev] = p;
+    }
+    *out = scratch_of_device[dev];
+    return QUEST_OK;
+}
+}  // namespace
+
+extern "C" size_t quest_gemm_noalloc_scratch_bytes(void) { return kScratchBytes; }
+
+extern "C" int quest_fused_matmul_dequantize_int4_int4t_noalloc(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                                const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                                const void *vec_a_mul, const void *vec_b_mul, int size_m,
+                                                                int size_k, int size_n, int dtype, void *stream) {
+    forget_stale_error();
+    const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
+    if (rc != QUEST_OK) return rc;
+    if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (size_m > 16) return QUEST_ERR_UNSUPPORTED;                                        // the decode sizes only
+    if (quest_gemm_workspace_bytes(size_m, size_k, size_n) > kScratchBytes) return QUEST_ERR_UNSUPPORTED;
+    void *work = nullptr;
+    const int got = scratch_here(&work);
+    if (got != QUEST_OK) return got;
+    const int out_kind = dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16;
+    const int split = launch_gemm_decode_splitk(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m,
+                                                size_k, size_n, work, kScratchBytes, (hipStream_t)stream);
     if (split != QUEST_ERR_UNSUPPORTED) return split;
     return gemm_launch(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m, size_k, size_n,
                        (hipStream_t)stream);
