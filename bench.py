@@ -48,9 +48,9 @@ FP6_MFMA_PEAK_TOPS = 10100.0
 # scaled by what the same counters read for calibration_stream() below (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0);
 # the runs are summarised under profiles/.
 TRAFFIC_SOURCE = ('constant from a separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this script, summarised in '
-                  'profiles/bench_gemm_M4096_K4096_N11008_and_quantize_8192x4096.md; not measured in this run')
-TRAFFIC_GEMM_BYTES = 343078377                 # placeholder until the counter run of this kernel: see TRAFFIC_GEMM_PLAN
-TRAFFIC_QUANTIZE_BYTES = 84236564
+                  'profiles/bench_gemm_e2m3_M4096_K4096_N11008_and_quantize_8192x4096.md; not measured in this run')
+TRAFFIC_GEMM_BYTES = 448892819                 # gemm_e2m3_kernel; of these 340.7 MB fetched (operands: 46.4 MB), 108.2 MB written
+TRAFFIC_QUANTIZE_BYTES = 84274484
 # what quest_e2m3_gemm_plan reported for M=4096 K=4096 N=11008 on 256 compute units when TRAFFIC_GEMM_BYTES was measured: the
 # figure depends on the schedule (which workgroup fetches what), so the line says `traffic_stale` when the plan has changed
 TRAFFIC_GEMM_PLAN = [256, 8, 0, 0, 256, 256, 6, 64]
@@ -615,6 +615,12 @@ def main():
     dec = bench_decode(_lib, dev)
     few_hundred = bench_decode(_lib, dev, ms=(128, 256, 384))
     fwd = None if args.no_forward else bench_forward(dev)
+    e2e = None
+    if not args.no_forward:
+        # the reference's end-to-end benchmark (gemm-quest/benchmarks/bench_e2e.py) at its largest batch: the 1600M model,
+        # 8 x 512 tokens; every batch size: python -m quest_amd.bench_e2e
+        from quest_amd import bench_e2e
+        e2e = bench_e2e.get_timing('1600m', (8,))[0]
     layer_sweep = None
     if args.layer_sweep:
         from quest_amd import bench_layer
@@ -645,6 +651,7 @@ def main():
     line = {
         'metric': 'INT4-GEMM TOPS + quantize GB/s at Llama-7B layer shapes, % MI355X roofline',
         'value': lin['tops'], 'unit': 'TOPS', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'untimed_steps': args.warmup + lin['untimed_replays'] * args.steps,
         'ms_per_step': lin['ms_per_step'], 'ms_per_step_eager_launches': lin['ms_per_step_eager'],
         'step_issue': f"one HIP graph of K steps, timed as K steps between two synchronisations after the W warm-up steps and "
                       f"{lin['untimed_replays']} untimed replays (60 ms: the clocks settle); median of five such timings, all in "
@@ -670,7 +677,8 @@ def main():
                                    'us_per_launch': lin['quant_alone_ms'] * 1e3,
                                    'GBs': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9,
                                    'frac_hbm': (4096 * 4096 * 2.5 + 4096 * 6) / (lin['quant_alone_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS},
-        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'few_hundred_tokens': few_hundred, 'forward': fwd, 'cpu_baseline': cpu,
+        'roofline': roofline, 'roofline_quantize': rq, 'decode': dec, 'few_hundred_tokens': few_hundred, 'forward': fwd, 'e2e_1600m_batch8': e2e,
+        'cpu_baseline': cpu,
     }
     if layer_sweep is not None:
         line['layer_sweep'] = layer_sweep
