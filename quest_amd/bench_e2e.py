@@ -137,7 +137,10 @@ def main():
     ap.add_argument('--matrix-path', choices=('fp6', 'int8'), default=None, help='force the GEMM path of large layers (default: harness.MATRIX_PATH)')
     ap.add_argument('--json', help='write the records to this file')
     ap.add_argument('--markdown', help='write the table to this file')
+    ap.add_argument('--min-k', type=int, default=None, help='shortest rows that take the FP6 path (default: harness.E2M3_MIN_K)')
     args = ap.parse_args()
+    if args.min_k is not None:
+        harness.E2M3_MIN_K = args.min_k
     if args.matrix_path is not None:
         harness.MATRIX_PATH = args.matrix_path
 

@@ -62,11 +62,22 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 // WPR waves share one row (32 blocks of 128 each); a workgroup holds one or two rows' worth of waves (small
 // workgroups: two-wave ones measured 3 % faster than four-wave ones for whole-wave rows, eight-wave ones 5 % slower).
-template <int WPR>
+// TL (E2M3 tiles staged through LDS, see the kernel): the workgroup holds eight consecutive rows (four when two or
+// three waves share a row), so that it owns whole 128-byte (64-byte) runs of every fragment it contributes to.
+template <int WPR, int G, bool TL>
 struct Shape {
-    static constexpr int kRows = WPR >= 3 ? 1 : 2;
+    static constexpr int kRowsPerWave = 32 / G;
+    static constexpr int kRows = !TL ? (WPR >= 3 ? 1 : 2) : WPR == 1 ? (8 / kRowsPerWave > 0 ? 8 / kRowsPerWave : 1) : 4;
     static constexpr int kWaves = WPR * kRows;
     static constexpr int kMinBlocks = kWaves <= 4 ? 4 : (16 / kWaves > 0 ? 16 / kWaves : 1);
+    static constexpr int kTileRows = kRows * kRowsPerWave;           // rows of a workgroup
+    // staging buffer: one position per (half of a k-step, k-step) of a row, the rows' 16-byte heads (8-byte tails) side
+    // by side; one spare chunk per position spreads the positions over the banks
+    static constexpr int kBlocks = G == 32 ? 32 * WPR : G;           // blocks of a row, rounded up
+    static constexpr int kPositions = 4 * kBlocks;
+    static constexpr int kHeadPitch = kTileRows * 16 + 16;
+    static constexpr int kTailPitch = kTileRows * 8 + 8;
+    static constexpr int kStageBytes = TL ? kPositions * (kHeadPitch + kTailPitch) : 16;
 };
 
 // What is applied to the input on its way into the transform (the producer the activation comes from):
@@ -100,15 +111,16 @@ __device__ __forceinline__ int group_sum_i(int v) {
 }
 
 // G = lanes of a half-wave per row (the row's blocks rounded up to a power of two): a wave holds 32 / G rows.
-template <int DT, int WPR, int G, int PRE>
-__global__ void __launch_bounds__(64 * Shape<WPR>::kWaves, Shape<WPR>::kMinBlocks)
+template <int DT, int WPR, int G, int PRE, bool TL>
+__global__ void __launch_bounds__((64 * Shape<WPR, G, TL>::kWaves), (Shape<WPR, G, TL>::kMinBlocks))
 hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ norm_w,
                               uint16_t *__restrict__ scale, uint32_t *__restrict__ packed, int32_t *__restrict__ row_sum,
                               uint16_t *__restrict__ x_had, uint16_t *__restrict__ pre_out, const uint16_t *add_in,
                               uint16_t *sum_out, uint8_t *__restrict__ tiles, int xcd_chunk, int K, int M, int ldx,
                               uint32_t entry_bits, float eps) {
     static_assert(WPR == 1 || G == 32, "rows shared by waves: whole waves");
-    constexpr int kRows = Shape<WPR>::kRows;
+    using Sh = Shape<WPR, G, TL>;
+    constexpr int kRows = Sh::kRows;
     constexpr int kRowsPerWave = 32 / G;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -196,7 +208,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
             for (int d = 0; d < 4; d++) ss = dot2_self<DT>(bq[s][d], ss);
         float ss_row = group_sum_f<G>(ss);
         if constexpr (WPR > 1) {                 // the row's waves add their parts in wave order: the same bits in each
-            __shared__ float part_pre[Shape<WPR>::kWaves];
+            __shared__ float part_pre[Sh::kWaves];
             if (lane == 0) part_pre[wave] = ss_row;
             __syncthreads();
             ss_row = 0.f;
@@ -262,8 +274,8 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
             }
     // lanes without a block transformed zeros: they add nothing
     float total = G == 32 ? wave_sum_dpp_f(sumsq) : group_sum_f<G>(sumsq);
-    __shared__ float part_sq[Shape<WPR>::kWaves];
-    __shared__ int part_sum[Shape<WPR>::kWaves];
+    __shared__ float part_sq[Sh::kWaves];
+    __shared__ int part_sum[Sh::kWaves];
     if constexpr (WPR > 1) {
         if (lane == 0) part_sq[wave] = total;
         __syncthreads();
@@ -294,6 +306,7 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
         const float sf_t = to_f32<DT>(s16);
         const float inv = quant_inv(sf_t);
         uint8_t *frag = tiles + ((size_t)(row >> 5) * (size_t)(K >> 6) + 2 * blk + h) * 1536;
+        __shared__ __attribute__((aligned(16))) uint8_t stage[Sh::kStageBytes];
         auto emit = [&](auto fast_tag) {
             constexpr bool kFast = decltype(fast_tag)::value;
 #pragma unroll
@@ -318,7 +331,13 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
                     }
                 }
                 const v6u r = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(__builtin_bit_cast(v32h, hp), 1.0f);
-                if (live) {
+                if constexpr (TL) {
+                    // position (g, h, block) of the row, this row's chunk in it
+                    const int pos = (2 * g + h) * Sh::kBlocks + blk;
+                    const int j = row_local * kRowsPerWave + n / G;
+                    *reinterpret_cast<uint4 *>(stage + pos * Sh::kHeadPitch + j * 16) = make_uint4(r[0], r[1], r[2], r[3]);
+                    *reinterpret_cast<uint2 *>(stage + Sh::kPositions * Sh::kHeadPitch + pos * Sh::kTailPitch + j * 8) = make_uint2(r[4], r[5]);
+                } else if (live) {
                     const int slot = 32 * g + (row & 31);
                     *reinterpret_cast<uint4 *>(frag + slot * 16) = make_uint4(r[0], r[1], r[2], r[3]);
                     *reinterpret_cast<uint2 *>(frag + 1024 + slot * 8) = make_uint2(r[4], r[5]);
@@ -327,6 +346,30 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
         };
         // degenerate rows (scale zero, Inf, NaN or outside the fast range) take the clamping form, as the nibbles do
         if (__builtin_amdgcn_ballot_w64(row < M && !quant_fast_ok(sf_t)) == 0) emit(std::true_type{}); else emit(std::false_type{});
+        if constexpr (TL) {
+            // The workgroup's rows are kTileRows consecutive slots of one row block: for every position their heads are
+            // one contiguous run of the fragment (128 bytes for eight rows) and their tails another, written by
+            // neighbouring lanes.  Rows past M inside the last row block are padding and are written like any other.
+            __syncthreads();
+            constexpr int kTR = Sh::kTileRows;
+            const int row0 = vb * kTR;
+            const int m_pad = (M + 31) & ~31;
+            const size_t frag0 = (size_t)(row0 >> 5) * (size_t)(K >> 6);
+            for (int u = threadIdx.x; u < Sh::kPositions * kTR; u += 64 * Sh::kWaves) {
+                const int pos = u / kTR, c = u % kTR;
+                const int gg = pos / (2 * Sh::kBlocks), hh = (pos / Sh::kBlocks) & 1, bb = pos % Sh::kBlocks;
+                if (bb < (K >> 7) && row0 + c < m_pad)
+                    *reinterpret_cast<uint4 *>(tiles + (frag0 + 2 * bb + hh) * 1536 + (32 * gg + (row0 & 31) + c) * 16) =
+                        *reinterpret_cast<const uint4 *>(stage + pos * Sh::kHeadPitch + c * 16);
+            }
+            for (int u = threadIdx.x; u < Sh::kPositions * kTR / 2; u += 64 * Sh::kWaves) {
+                const int pos = u / (kTR / 2), c = 2 * (u % (kTR / 2));
+                const int gg = pos / (2 * Sh::kBlocks), hh = (pos / Sh::kBlocks) & 1, bb = pos % Sh::kBlocks;
+                if (bb < (K >> 7) && row0 + c < m_pad)
+                    *reinterpret_cast<uint4 *>(tiles + (frag0 + 2 * bb + hh) * 1536 + 1024 + (32 * gg + (row0 & 31) + c) * 8) =
+                        *reinterpret_cast<const uint4 *>(stage + Sh::kPositions * Sh::kHeadPitch + pos * Sh::kTailPitch + c * 8);
+            }
+        }
     }
     if (packed == nullptr && row_sum == nullptr) return;      // uniform over the workgroup
 
@@ -433,18 +476,28 @@ struct Args {
     hipStream_t st;
 };
 
-template <int DT, int WPR, int G, int PRE>
-static void launch_shape(const Args &a) {
-    constexpr int rows = hq::Shape<WPR>::kRows * (32 / G);        // rows per workgroup
+template <int DT, int WPR, int G, int PRE, bool TL>
+static void launch_shape_as(const Args &a) {
+    using Sh = hq::Shape<WPR, G, TL>;
+    constexpr int rows = Sh::kTileRows;                            // rows per workgroup
     int grid = (a.M + rows - 1) / rows, xcd_chunk = 0;
     if (a.tiles != nullptr) {                                     // see the kernel: a contiguous range of rows per XCD
         xcd_chunk = (grid + 7) / 8;
         grid = 8 * xcd_chunk;
     }
-    hq::hadamard_quantize_mfma_kernel<DT, WPR, G, PRE><<<dim3(grid), dim3(64 * hq::Shape<WPR>::kWaves), 0, a.st>>>(
+    hq::hadamard_quantize_mfma_kernel<DT, WPR, G, PRE, TL><<<dim3(grid), dim3(64 * Sh::kWaves), 0, a.st>>>(
         (const uint16_t *)a.x, (const uint16_t *)a.norm_w, (uint16_t *)a.scale, (uint32_t *)a.packed, a.row_sum,
         (uint16_t *)a.x_had, (uint16_t *)a.pre_out, (const uint16_t *)a.add_in, (uint16_t *)a.sum_out, a.tiles, xcd_chunk,
         a.K, a.M, a.ldx, a.bits, a.eps);
+}
+
+// Tiles go through the workgroup's LDS where a workgroup of eight (four) rows fits: rows of 8 to 96 blocks.
+template <int DT, int WPR, int G, int PRE>
+static void launch_shape(const Args &a) {
+    if constexpr (WPR <= 3 && G >= 8) {
+        if (a.tiles != nullptr) return launch_shape_as<DT, WPR, G, PRE, true>(a);
+    }
+    launch_shape_as<DT, WPR, G, PRE, false>(a);
 }
 
 // rows of up to 32 blocks: one wave holds 32 / G of them

@@ -22,6 +22,7 @@ WEIGHT_HADAMARD_SCALE = 2. ** -3.5      # utils.py:39
 # INT8 kernels on packed nibbles.  Both give the same bits.
 MATRIX_PATH = 'fp6'
 E2M3_MIN_TILES = 66                     # 256 x 256 output tiles from which the FP6 kernel is the faster one
+E2M3_MIN_K = 2048                       # shortest rows that take it (see prefers_e2m3)
 
 
 def prefers_e2m3(m: int, k: int, n: int) -> bool:
@@ -30,10 +31,11 @@ def prefers_e2m3(m: int, k: int, n: int) -> bool:
     2048 to 13824 and M from 256 to 16384, the FP6 kernel wins from 66 tiles on (M = 1536 at N = 4096, M = 512 at
     N = 11008, M = 3072 at N = 2048) and loses below 64."""
     tiles = ((m + 255) // 256) * ((n + 255) // 256)
-    # K >= 2048: with shorter rows the GEMM is mostly epilogue either way, and what the FP6 kernel gains there (10-15 % on
-    # random codes) the activation kernels lose again writing tiles (scattered 16-byte pieces) instead of packed rows --
-    # measured on the 12-layer d = 1024 model: 6.17 ms per forward with tiles everywhere against 5.95 ms without
-    return (MATRIX_PATH == 'fp6' and k % 128 == 0 and 2048 <= k <= 65536 and tiles >= E2M3_MIN_TILES and m * n <= (1 << 30))
+    # E2M3_MIN_K: with shorter rows the GEMM is mostly epilogue either way and the tile-writing activation kernels are a
+    # little slower than the row-writing ones (12.0 against 10.2 us at [16384, 1024]) -- measured on the 12-layer
+    # d = 1024 model at 32 x 512 tokens: 6.01 ms per forward with the FP6 path from K = 1024 on, 5.79 ms from K = 2048 on
+    # (its K = 2816 layers), 5.80 ms without it; the 1600M model (K = 2560, 6912) gains 9 %
+    return (MATRIX_PATH == 'fp6' and k % 128 == 0 and E2M3_MIN_K <= k <= 65536 and tiles >= E2M3_MIN_TILES and m * n <= (1 << 30))
 
 
 def weight_tiles(w_int_packed: torch.Tensor) -> torch.Tensor:
