@@ -423,3 +423,73 @@ def test_fake_quant_linear_equals_packed_linear_in_exact_arithmetic():
     lhs = (2 * c + a.sum(-1, keepdim=True) + (b.sum(-1, keepdim=True) + 128).t()).double()
     got = lhs * (0.5 * xstep.double() * wstep.double().t())
     assert torch.allclose(got, want.double(), rtol=1e-4, atol=1e-6)
+
+
+# --------------------------------------------------------------------------- E2M3 tiles (the FP6 GEMM's operand form)
+def test_e2m3_values_are_the_ocp_fp6_table():
+    """OCP Microscaling Formats (MX) v1.0, FP6 E2M3: bias 1, no Inf / NaN; max normal 7.5, min normal 1.0, max
+    subnormal 0.875, min subnormal 0.125 -- and the whole table built from exact fractions, not from the oracle's
+    formula."""
+    v = qo.e2m3_value(torch.arange(64))
+    assert float(v[0b011111]) == 7.5 and float(v[0b001000]) == 1.0 and float(v[0b000111]) == 0.875 and float(v[0b000001]) == 0.125
+    assert float(v[0b100100]) == -0.5 and float(v[0b111111]) == -7.5 and float(v[0]) == 0.0 and float(v[0b010000]) == 2.0
+    for bits in range(64):
+        e, m = (bits >> 3) & 3, bits & 7
+        mag = Fraction(m, 8) if e == 0 else Fraction(8 + m, 8) * Fraction(2) ** (e - 1)
+        assert Fraction(float(v[bits])) == (-mag if bits & 32 else mag)
+    pos = v[:32]
+    assert bool((pos[1:] > pos[:-1]).all())                       # monotone in the magnitude bits
+
+
+def test_e2m3_code_patterns_hold_q_plus_half():
+    """Every INT4 code has exactly one pattern, its value is q + 1/2, and the patterns are the eight magnitudes
+    {0.5, 1.5, ..., 7.5} with the sign bit for negative codes (q and -q - 1 share a magnitude)."""
+    q = torch.arange(-8, 8)
+    bits = qo.e2m3_bits_of_code(q)
+    assert torch.equal(qo.e2m3_value(bits), q.double() + 0.5)
+    assert bits[8:].tolist() == [0b000100, 0b001100, 0b010010, 0b010110, 0b011001, 0b011011, 0b011101, 0b011111]
+    assert torch.equal(bits[:8].flip(0), bits[8:] | 32)
+    table = qo.e2m3_value(torch.arange(64))
+    for c in q.tolist():
+        assert int((table == c + 0.5).sum()) == 1
+
+
+def test_e2m3_tiles_layout_bit_by_bit():
+    """One nonzero code at a time: its six bits land where the layout says -- fragment (row / 32, k / 64), lane
+    32 * ((k % 64) / 32) + row % 32, bit 6 * (k % 32) of the lane's 24 bytes, whose first 16 sit at byte 16 * lane and
+    whose last 8 at byte 1024 + 8 * lane of the fragment's 1536.  Everything else holds the pattern of code 0 there."""
+    rows, k = 40, 192
+    base = qo.e2m3_tiles_encode(torch.zeros(rows, k, dtype=torch.int8))
+    assert base.numel() == 2 * 3 * 1536
+    zero_pat = 0b000100                                           # 0 + 1/2
+    for (r, c, code) in [(0, 0, 7), (0, 5, -8), (31, 63, 3), (33, 64, -1), (39, 191, 6), (17, 100, -5), (5, 21, 2), (6, 26, -3)]:
+        x = torch.zeros(rows, k, dtype=torch.int8)
+        x[r, c] = code
+        t = qo.e2m3_tiles_encode(x)
+        diff = (t != base).nonzero().flatten().tolist()
+        frag, lane, bit = (r // 32) * (k // 64) + c // 64, 32 * ((c % 64) // 32) + r % 32, 6 * (c % 32)
+        pat = {7: 0b011111, -8: 0b111111, 3: 0b010110, -1: 0b100100, 6: 0b011101, -5: 0b111001, 2: 0b010010, -3: 0b110010}[code]
+        want = set()
+        for b in range(6):
+            if ((pat ^ zero_pat) >> b) & 1:
+                byte_in_lane = (bit + b) // 8
+                want.add(frag * 1536 + (16 * lane + byte_in_lane if byte_in_lane < 16 else 1024 + 8 * lane + byte_in_lane - 16))
+        assert set(diff) == want, (r, c, code)
+        # and the bits themselves
+        lane_bytes = torch.cat((t[frag * 1536 + 16 * lane:frag * 1536 + 16 * lane + 16], t[frag * 1536 + 1024 + 8 * lane:frag * 1536 + 1024 + 8 * lane + 8]))
+        word = int.from_bytes(bytes(lane_bytes.tolist()), 'little')
+        assert (word >> bit) & 63 == pat
+
+
+def test_e2m3_tiles_round_trip_and_padding():
+    g = torch.Generator().manual_seed(5)
+    for rows, k in [(1, 64), (32, 128), (45, 256), (100, 64)]:
+        x = torch.randint(-8, 8, (rows, k), generator=g, dtype=torch.int8)
+        t = qo.e2m3_tiles_encode(x)
+        assert t.numel() == ((rows + 31) // 32) * (k // 64) * 1536
+        assert torch.equal(qo.e2m3_tiles_decode(t, rows, k), x.double() + 0.5)
+        # a product of decoded tiles is sum (qa + 1/2)(qb + 1/2): twice it is 2 C + sum qa + sum qb + K / 2
+        y = torch.randint(-8, 8, (7, k), generator=g, dtype=torch.int8)
+        s = qo.e2m3_tiles_decode(t, rows, k) @ qo.e2m3_tiles_decode(qo.e2m3_tiles_encode(y), 7, k).T
+        c = x.double() @ y.double().T
+        assert torch.equal(2 * s, 2 * c + x.double().sum(1, keepdim=True) + y.double().sum(1)[None, :] + k / 2)
