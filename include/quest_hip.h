@@ -268,8 +268,8 @@ int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_tiles, const v
 /*
  * Diagnostic (host only, nothing is launched): how quest_fused_matmul_dequantize_e2m3 divides a shape among the
  * workgroups of a device with `cus` compute units.  plan[0..7] = workgroups, scheduling groups (one per XCD when 8),
- * tiles per token tile when every workgroup gets exactly one (else 0), whether the groups divide the token tiles (1) or
- * the channel units (0), tile rows, tile channels at most, LDS slots, k per slot.  A measured figure that depends on
+ * tiles per token tile when every workgroup gets exactly one (else 0), how many ways the groups divide the token tiles
+ * (0 or 1: not at all, each group takes a slice of the channel units; g: a g x groups / g grid of groups), tile rows, tile channels at most, LDS slots, k per slot.  A measured figure that depends on
  * the schedule (HBM traffic per launch) is only valid while this plan is the one it was measured under.
  */
 int quest_e2m3_gemm_plan(int size_m, int size_k, int size_n, int cus, int *plan);

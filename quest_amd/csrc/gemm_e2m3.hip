@@ -40,6 +40,7 @@ constexpr int kFrags = 16;                       // per slot: 8 token row blocks
 constexpr int kHeadsB = kFrags * kHeadB;         // heads first, tails after them
 constexpr int kStageB = kFrags * kFragB;         // 24 KiB
 constexpr int kStages = 6;
+constexpr int kTokSplit = -1;                    // XCD groups along the tokens: chosen per shape (see make_schedule)
 constexpr int kLoads = 6;                        // direct loads per wave per step: four heads, two pairs of tails
 constexpr int kVecParB = 2 * kRows * 2;          // a_mul of the tile's tokens and b_mul of its channels, 16-bit
 constexpr int kVecOff = kStages * kStageB;
@@ -433,7 +434,7 @@ template <bool GLU>
 static int launch_e2m3(int dtype, void *out, const uint8_t *a, const uint8_t *b, const void *a_mul, const void *b_mul, int M,
                        int K, int N, int cus, hipStream_t st) {
     long grid = 0;
-    const Schedule sch = make_schedule(M, N, e2m3::kMaxUnits, 1, cus, &grid);
+    const Schedule sch = make_schedule(M, N, e2m3::kMaxUnits, 1, cus, &grid, e2m3::kTokSplit);
     if (dtype == QUEST_DTYPE_BF16)
         e2m3::gemm_e2m3_kernel<OUT_BF16, GLU><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
             out, a, b, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
@@ -493,7 +494,7 @@ extern "C" int quest_e2m3_gemm_plan(int size_m, int size_k, int size_n, int cus,
     if (!plan) return QUEST_ERR_NULL_POINTER;
     if (size_m <= 0 || size_n <= 0 || size_k <= 0 || (size_k & 127) || cus <= 0) return QUEST_ERR_BAD_SHAPE;
     long grid = 0;
-    const Schedule sch = make_schedule(size_m, size_n, e2m3::kMaxUnits, 1, cus, &grid);
+    const Schedule sch = make_schedule(size_m, size_n, e2m3::kMaxUnits, 1, cus, &grid, e2m3::kTokSplit);
     const int v[8] = {(int)grid, sch.groups, sch.row_tiles, sch.by_tokens, e2m3::kRows, 32 * e2m3::kMaxUnits, e2m3::kStages, 64};
     for (int i = 0; i < 8; i++) plan[i] = v[i];
     return QUEST_OK;

@@ -11,7 +11,8 @@ struct Schedule {
     int units;          // channel units of 32
     int groups;         // channel super-groups (one per XCD when the grid allows)
     int row_tiles;      // > 0: one tile per workgroup, this many per token tile of a group (0: contiguous runs of cells)
-    int by_tokens;      // the groups divide the token tiles among them (and each takes all channel units) instead of the units
+    int by_tokens;      // how many ways the groups divide the token tiles (1: every group takes all token tiles and 1/groups of the
+                        // channel units; groups: the other way round; in between: a groups_t x groups / groups_t grid of groups)
 };
 
 struct Cursor {          // walks a workgroup's run of cells tile by tile, stage by stage (no divisions)
@@ -52,12 +53,18 @@ __device__ __forceinline__ void cursor_begin(const Schedule &sch, Cursor &cc) {
     // by_tokens -- a slice of the token tiles and all units: whichever operand is the smaller one is then the one every
     // XCD fetches whole (and keeps in its L2), and the larger one is fetched once in total.
     int ug0 = 0, ug1 = sch.units, tt_lo = 0, tt_hi = sch.tiles_t;
-    if (sch.by_tokens) {
-        tt_lo = __builtin_amdgcn_readfirstlane((int)(((long)grp * sch.tiles_t) / sch.groups));
-        tt_hi = __builtin_amdgcn_readfirstlane((int)(((long)(grp + 1) * sch.tiles_t) / sch.groups));
-    } else {
-        ug0 = __builtin_amdgcn_readfirstlane((int)(((long)grp * sch.units) / sch.groups));
-        ug1 = __builtin_amdgcn_readfirstlane((int)(((long)(grp + 1) * sch.units) / sch.groups));
+    {
+        const int gt_n = sch.by_tokens > 0 ? sch.by_tokens : 1;          // groups along the tokens
+        const int gu_n = sch.groups / gt_n;                              // groups along the channels
+        const int gt = grp % gt_n, gu = grp / gt_n;
+        if (gt_n > 1) {
+            tt_lo = __builtin_amdgcn_readfirstlane((int)(((long)gt * sch.tiles_t) / gt_n));
+            tt_hi = __builtin_amdgcn_readfirstlane((int)(((long)(gt + 1) * sch.tiles_t) / gt_n));
+        }
+        if (gu_n > 1) {
+            ug0 = __builtin_amdgcn_readfirstlane((int)(((long)gu * sch.units) / gu_n));
+            ug1 = __builtin_amdgcn_readfirstlane((int)(((long)(gu + 1) * sch.units) / gu_n));
+        }
     }
     cc.nug = ug1 - ug0;
     cc.ug0 = ug0;
@@ -89,7 +96,7 @@ __device__ __forceinline__ void cursor_begin(const Schedule &sch, Cursor &cc) {
 
 // Host side: the schedule and the grid for M tokens x N channels with tiles of up to max_units units and
 // wg_per_cu persistent workgroups on each of the device's `cus` compute units.
-inline Schedule make_schedule(int M, int N, int max_units, int wg_per_cu, int cus, long *grid_out) {
+inline Schedule make_schedule(int M, int N, int max_units, int wg_per_cu, int cus, long *grid_out, int tok_split = 0) {
     Schedule sch;
     sch.tiles_t = (M + kBigTileRows - 1) / kBigTileRows;
     sch.units = (N + 31) / 32;
@@ -104,7 +111,31 @@ inline Schedule make_schedule(int M, int N, int max_units, int wg_per_cu, int cu
     // (measured +4..7 % at M = 16384 with N = 1024..5632; no difference at M = 4096, N = 11008 either way).
     if (M > N && grid % 8 == 0 && sch.tiles_t >= 8) {
         sch.groups = 8;
-        sch.by_tokens = 1;
+        sch.by_tokens = 8;
+    }
+    // tok_split < 0: the grid of groups (1 x 8, 2 x 4, 4 x 2 or 8 x 1) that fetches least from behind the L2s.  The
+    // workgroups of a group work on T token tiles x C channel ranges at a time (T C = workgroups per group) and one such
+    // round fetches T + C operand tiles of equal size; splitting the token tiles g ways makes T = tiles_t / g.  At
+    // M = 4096, N = 11008: 16 + 2 tiles as 1 x 8, 8 + 4 as 2 x 4 (a third less traffic, the same time); at M = 8192:
+    // 32 + 1 against 8 + 4 as 4 x 2 (238 -> 217 us).  Only where every workgroup has several full tiles to walk.
+    if (tok_split < 0 && grid % 8 == 0 && sch.units >= 8 && cells >= 2L * max_units * grid) {
+        const long per_grp = grid / 8;
+        long best_cost = 0;
+        int best = 0;
+        for (int g = 1; g <= 8; g *= 2) {
+            if (sch.tiles_t % g != 0 || sch.units < (long)max_units * (8 / g)) continue;
+            long t = sch.tiles_t / g;
+            if (t > per_grp) t = per_grp;
+            const long c = per_grp / t > 1 ? per_grp / t : 1;
+            if (best == 0 || t + c < best_cost) { best = g; best_cost = t + c; }
+        }
+        if (best > 0) {
+            sch.groups = 8;
+            sch.by_tokens = best > 1 ? best : 0;
+        }
+    } else if (!sch.by_tokens && sch.groups == 8 && tok_split > 1 && sch.tiles_t % tok_split == 0 &&
+               sch.units >= 2L * max_units * (8 / tok_split) && cells >= 2L * max_units * grid) {
+        sch.by_tokens = tok_split;
     }
     if (!sch.by_tokens) {
         // few cells per workgroup: one tile each, cut along the channel units of single token tiles (see cursor_begin)
