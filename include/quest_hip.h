@@ -144,7 +144,10 @@ int quest_hadamard128(void *y, const void *x, int group_size, int batch_size, fl
  * Which arithmetic runs depends on (group_size, had_scale, dtype) only, never on batch_size or on where the buffers
  * lie: a had_scale the dtype holds exactly (181/2048) with group_size <= 32768 is the product with the +-had_scale
  * matrix on the matrix cores, fp32 accumulation, as the reference states the activation transform; any other factor
- * (2^-3.5, the weight-side one), and rows over 32768, are fp32 butterflies followed by one multiplication.  The two
+ * (2^-3.5, the weight-side one), and rows over 32768, are fp32 butterflies followed by one multiplication.  Without a
+ * transform (had_scale == 0) rows of whole blocks of 128 up to 32768 run on the same matrix-core kernel with the
+ * multiplications left out (the values only change lanes), other rows on the row kernel; the two differ in the order
+ * of the fp32 sum of squares only (the scale may come out one ulp apart on rare rows).  The two transforms
  * agree to fp32 summation noise (<= 1e-3 relative, the transform's stated bar), so that a value on a rounding boundary
  * of the dtype may come out one ulp apart and its code one level apart: codes are reproducible for a given shape,
  * factor and dtype, not across the two.  Given the transformed tensor and the scale, codes and row sums are exactly
@@ -284,9 +287,9 @@ int quest_fused_matmul_dequantize_swiglu_e2m3(void *mat_d, const void *a_tiles, 
  * quest_hadamard_quantize_int4 writing the codes as E2M3 tiles (x_tiles, quest_e2m3_tiles_bytes(batch_size,
  * group_size) bytes; rows past batch_size in the last row block are left unwritten: the GEMM never uses what it
  * computes from them).  The tiles hold exactly the codes the packed output would: x_int_packed and x_int_row_sum may
- * be asked for as well.  Only the matrix-core form of the transform writes tiles: had_scale must be exactly
- * representable in dtype (181/2048 is) and group_size <= 32768, QUEST_ERR_UNSUPPORTED otherwise (the caller then
- * quantises to packed codes and converts them with quest_int4_to_e2m3_tiles).
+ * be asked for as well.  Only the matrix-core kernel writes tiles: had_scale must be exactly representable in dtype
+ * (181/2048 is) or 0 (no transform), group_size % 128 == 0 and <= 32768; QUEST_ERR_UNSUPPORTED otherwise (the caller
+ * then quantises to packed codes and converts them with quest_int4_to_e2m3_tiles).
  */
 int quest_hadamard_quantize_e2m3(const void *x, void *scale, void *x_tiles, uint8_t *x_int_packed,
                                  int32_t *x_int_row_sum, void *x_had, int group_size, int batch_size, float had_scale,

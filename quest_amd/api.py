@@ -423,6 +423,7 @@ def fused_matmul_dequantize_e2m3(
 
 
 QUEST_ERR_UNSUPPORTED = -5
+QUEST_ERR_BAD_SHAPE = -2
 
 
 def hadamard_quantize_e2m3(
@@ -436,7 +437,8 @@ def hadamard_quantize_e2m3(
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """`hadamard_quantize_int4` with the codes written as E2M3 tiles (one pass over x).  x_int_packed / x_int_row_sum,
     if given, receive the packed form of the same codes as well.  Shapes the matrix-core kernel does not take (no
-    transform, the weight-side factor, rows over 32768) are quantised to packed codes first and converted.
+    transform on rows that are not whole blocks of 128, the weight-side factor, rows over 32768) are quantised to packed
+    codes first and converted.
     Returns (scale, x_tiles)."""
     m, k = x.shape
     if scale is None:
@@ -452,7 +454,7 @@ def hadamard_quantize_e2m3(
     with torch.cuda.device(dev):
         rc = _lib.load().quest_hadamard_quantize_e2m3(ptr(x), ptr(scale), ptr(x_tiles), ptr(x_int_packed), ptr(x_int_row_sum),
                                                       ptr(x_had), k, m, float(hadamard_scale), DTYPE_CODE[x.dtype], stream_of(x))
-    if rc == QUEST_ERR_UNSUPPORTED:
+    if rc == QUEST_ERR_UNSUPPORTED or (rc == QUEST_ERR_BAD_SHAPE and hadamard_scale == 0. and k % 64 == 0):
         _, packed, _ = hadamard_quantize_int4(x, scale, x_int_packed, x_int_row_sum, x_had, hadamard_scale=hadamard_scale)
         int4_to_e2m3_tiles(packed, x_tiles)
     else:

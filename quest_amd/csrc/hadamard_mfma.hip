@@ -243,35 +243,52 @@ hadamard_quantize_mfma_kernel(const uint16_t *__restrict__ x, const uint16_t *__
         }
     }
 
-    // ---- Hadamard: 8 k-steps x 4 row tiles
-    v16f acc[4];
-#pragma unroll
-    for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[mt][r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < 8; s++) {
-        const v4i b = __builtin_bit_cast(v4i, bq[s]);
-#pragma unroll
-        for (int mt = 0; mt < 4; mt++) {
-            const int neg = ((mt & 1) & ((s >> 1) & 1)) ^ (((mt >> 1) & 1) & ((s >> 2) & 1));
-            acc[mt] = mfma_h<DT>(hv[s & 1][neg], b, acc[mt]);
-        }
-    }
-
-    // ---- round to the dtype (the transform's output exists only in dtype), sum of squares
+    // ---- Hadamard: 8 k-steps x 4 row tiles; then round to the dtype (the transform's output exists only in dtype) and
+    // sum the squares.  entry_bits == 0: no transform -- the loaded chunks are the outputs already and only have to
+    // change lanes: lane (n, h) loaded the chunks whose k has bit 3 equal to h and the code below wants those whose bit 2
+    // is h, so the two half-waves trade half of every chunk (nothing is multiplied: NaN and Inf stay where they are).
     uint32_t yb[4][8];                          // [mt][q * 2 + pair]: outputs 32 mt + 8 q + 4 h + {0,1} / {2,3}
     float sumsq = 0.f;
+    if (entry_bits == 0) {                      // uniform
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-        for (int q = 0; q < 4; q++)
+        for (int s = 0; s < 8; s++)
 #pragma unroll
             for (int p = 0; p < 2; p++) {
-                const uint32_t w = pack2_rne<DT>(acc[mt][q * 4 + 2 * p], acc[mt][q * 4 + 2 * p + 1]);
-                yb[mt][q * 2 + p] = w;
-                sumsq = dot2_self<DT>(w, sumsq);            // both squares straight from the packed pair
+                // outputs 16 s + 8 (q & 1) + 4 h + 2 p + {0, 1}: pair 2 h + p of the chunk held by the half-wave q & 1
+                const auto sw = __builtin_amdgcn_permlane32_swap(bq[s][p], bq[s][2 + p], false, false);
+#pragma unroll
+                for (int qo = 0; qo < 2; qo++) {
+                    const uint32_t w = sw[qo];
+                    yb[s >> 1][(2 * (s & 1) + qo) * 2 + p] = w;
+                    sumsq = dot2_self<DT>(w, sumsq);
+                }
             }
+    } else {
+        v16f acc[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mt][r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const v4i b = __builtin_bit_cast(v4i, bq[s]);
+#pragma unroll
+            for (int mt = 0; mt < 4; mt++) {
+                const int neg = ((mt & 1) & ((s >> 1) & 1)) ^ (((mt >> 1) & 1) & ((s >> 2) & 1));
+                acc[mt] = mfma_h<DT>(hv[s & 1][neg], b, acc[mt]);
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int p = 0; p < 2; p++) {
+                    const uint32_t w = pack2_rne<DT>(acc[mt][q * 4 + 2 * p], acc[mt][q * 4 + 2 * p + 1]);
+                    yb[mt][q * 2 + p] = w;
+                    sumsq = dot2_self<DT>(w, sumsq);            // both squares straight from the packed pair
+                }
+    }
     // lanes without a block transformed zeros: they add nothing
     float total = G == 32 ? wave_sum_dpp_f(sumsq) : group_sum_f<G>(sumsq);
     __shared__ float part_sq[Sh::kWaves];
@@ -553,7 +570,8 @@ int launch_hadamard_quantize_mfma(int pre, const void *x, const void *norm_w, fl
                                   int32_t *row_sum, void *x_had, void *pre_out, int K, int M, float had_scale, int dtype,
                                   hipStream_t st, const void *add_in, void *sum_out, uint8_t *tiles) {
     uint32_t bits = 0;
-    if (K > 32768 || (K & 127) || had_scale <= 0.f || !representable16(had_scale, dtype, &bits)) return QUEST_ERR_UNSUPPORTED;
+    // (had_scale == 0: no transform; the kernel then only moves the chunks between lanes)
+    if (K > 32768 || (K & 127) || had_scale < 0.f || !representable16(had_scale, dtype, &bits)) return QUEST_ERR_UNSUPPORTED;
     const int ldx = pre == hq::kPreSiluMul ? 2 * K : K;
     if (!aligned(pre_out, 16) || !aligned(norm_w, 16)) return QUEST_ERR_UNSUPPORTED;
     if (add_in != nullptr && (pre != hq::kPreRmsNorm || sum_out == nullptr || !aligned(add_in, 16) || !aligned(sum_out, 16)))

@@ -220,11 +220,46 @@ def test_activation_tiles_degenerate_rows(quest, dtype):
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(64, 4096), (33, 1024), (70, 128), (5, 2816), (40, 11008), (130, 512), (3, 32768)])
+def test_no_transform_on_the_matrix_core_kernel(quest, dtype, shape):
+    """hadamard_scale = 0 with rows of whole blocks of 128: the matrix-core kernel without its multiplications (the
+    loaded chunks only change lanes).  The scale is the oracle's on x itself (one ulp: summation order), the codes are the
+    oracle's given that scale, bit for bit, degenerate elements included, and the tiles hold the same codes."""
+    m, k = shape
+    x = rand_act(m, k, dtype, 31)
+    if m > 4:
+        x[1] = 0
+        x[2, 5] = float('nan')
+        x[3, 7] = float('inf')
+        x[4, k - 1] = float('-inf')
+    x_had = torch.empty(m, k, dtype=dtype, device=DEV)
+    scale, packed, row_sum = quest.hadamard_quantize_int4(x.to(DEV), hadamard_scale=0., x_had=x_had)
+    assert torch.equal(bits(x_had.cpu()), bits(x))                           # nothing was multiplied
+    want_scale = qo.find_scale_int4(x)
+    ok = torch.isfinite(want_scale.float()).flatten() & (want_scale.float().flatten() != 0)
+    assert (bits(scale.cpu()) - bits(want_scale)).abs().flatten()[ok].max() <= 1
+    want_packed = torch.empty(m, k // 2, dtype=torch.uint8)
+    want_sum = torch.empty(m, 1, dtype=torch.int32)
+    qo.quantize_int4(x.clone(), scale.cpu(), None, want_packed, want_sum, False)
+    clean = torch.ones(m, dtype=torch.bool)
+    if m > 4:
+        clean[1:5] = False              # scale 0, NaN or Inf: what the codes are is this build's definition, pinned by
+                                        # the unfused kernel below (and by the degenerate-row tests of the configurations)
+    assert torch.equal(packed.cpu()[clean], want_packed[clean]) and torch.equal(row_sum.cpu()[clean], want_sum[clean])
+    unfused = torch.empty(m, k // 2, dtype=torch.uint8, device=DEV)
+    quest.quantize_int4(x.to(DEV), scale, None, unfused, None, False)
+    assert torch.equal(packed, unfused)
+    _, tiles = quest.hadamard_quantize_e2m3(x.to(DEV), hadamard_scale=0.)
+    assert torch.equal(qo.e2m3_tiles_decode(tiles.cpu(), m, k), qo.unpack_int4(packed.cpu()).double() + .5)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
 def test_tiles_fall_back_without_the_matrix_core_transform(quest, dtype):
-    """No transform (hadamard_scale = 0) and the weight-side factor: quantised to packed codes, then converted."""
-    m, k = 40, 384
-    x = rand_act(m, k, dtype, 23).to(DEV)
-    for hs in (0., 2. ** -3.5):
+    """The weight-side factor, and no transform on rows that are not whole blocks of 128: quantised to packed codes by
+    the row kernel, then converted."""
+    m = 40
+    for k, hs in ((384, 2. ** -3.5), (320, 0.), (64, 0.)):
+        x = rand_act(m, k, dtype, 23).to(DEV)
         _, packed, _ = quest.hadamard_quantize_int4(x, hadamard_scale=hs)
         _, tiles = quest.hadamard_quantize_e2m3(x, hadamard_scale=hs)
         assert torch.equal(qo.e2m3_tiles_decode(tiles.cpu(), m, k), qo.unpack_int4(packed.cpu()).double() + .5)
