@@ -126,6 +126,34 @@ def test_graph_replay_and_noop(llama):
     assert y.shape == (2, 1, cfg.vocab_size) and torch.isfinite(y).all()
 
 
+def test_wide_blocks_take_the_fp6_path_and_match_the_int8_path(llama):
+    """Two blocks of the 1600M model's width (d = 2560, hidden 6912) at 4 x 512 tokens: every projection is long and
+    wide enough for the FP6 kernel on E2M3 tiles.  The forward equals, bit for bit, the same model forced onto the
+    packed-nibble INT8 kernels (both GEMM paths give the same bits and the activation kernels the same codes), is
+    deterministic, and replays from a HIP graph."""
+    from quest_amd import harness
+    cfg = llama.LlamaConfig(n_layer=2, n_embd=2560, n_head=20, vocab_size=2048, sequence_length=512)
+    ids = torch.randint(0, cfg.vocab_size, (4, 512), generator=torch.Generator().manual_seed(3)).to(DEV)
+    assert harness.prefers_e2m3(4 * 512, 2560, 3 * 2560) and harness.prefers_e2m3(4 * 512, 6912, 2560)
+    out = {}
+    try:
+        for path in ('fp6', 'int8'):
+            harness.MATRIX_PATH = path
+            torch.manual_seed(0)
+            model = llama.Llama(cfg).to(torch.bfloat16).to(DEV).eval()
+            llama.quantize_model(model, 'int4', use_hadamard=True, fuse_gate_up=True, fuse_producers=True)
+            with torch.inference_mode():
+                out[path] = model.hidden_states(ids).clone()
+                assert torch.equal(out[path], model.hidden_states(ids))
+            if path == 'fp6':
+                assert llama.bench_forward(model, 4, 512, n_warmup=2, n_iter=2)['graph_matches_eager']
+            del model
+    finally:
+        harness.MATRIX_PATH = 'fp6'
+    assert torch.isfinite(out['fp6'].float()).all()
+    assert torch.equal(out['fp6'], out['int8'])
+
+
 def test_packed_checkpoint_serves_the_same_logits(llama, tmp_path):
     from quest_amd import checkpoint
     model, cfg, _ = build(llama, torch.bfloat16, seed=5)
