@@ -71,6 +71,13 @@ def test_activation_kernel_8192x4096(quest):
     s3, p3, r3 = quest.hadamard_quantize_int4(gx)
     assert torch.equal(bits(scale.cpu()), bits(s3.cpu())) and torch.equal(packed, p3) and torch.equal(row_sum, r3)
 
+    # the same codes as E2M3 tiles, over the whole tensor: byte for byte the conversion of the packed output (which
+    # tests/test_gpu_e2m3.py holds against the oracle's encoding); m is whole row blocks, so there is no padding
+    s4, tiles = quest.hadamard_quantize_e2m3(gx)
+    assert torch.equal(bits(s4.cpu()), bits(scale.cpu()))
+    assert torch.equal(tiles, quest.int4_to_e2m3_tiles(packed))
+    assert torch.equal(qo.e2m3_tiles_decode(tiles[:2 * (k // 64) * 1536].cpu(), 64, k), qo.unpack_int4(packed[:64].cpu()).double() + .5)
+
     # the oracle on sampled rows: transform within tolerance, codes bit for bit given the kernel's transform and scale
     rows = torch.randperm(m, generator=torch.Generator().manual_seed(1))[:96]
     xs = x[rows]
@@ -103,6 +110,13 @@ def test_activation_tensor_of_2_gib_and_more(quest):
         s2, p2, r2 = quest.hadamard_quantize_int4(x[lo:hi])
         assert torch.equal(bits(scale[lo:hi].cpu()), bits(s2.cpu())), (lo, hi)
         assert torch.equal(packed[lo:hi], p2) and torch.equal(row_sum[lo:hi], r2), (lo, hi)
+    # the tiles of the same tensor (the second launch continues in the row block after the cut): byte for byte the
+    # conversion of the packed codes, over every whole row block
+    s6, tiles = quest.hadamard_quantize_e2m3(x)
+    assert torch.equal(bits(s6.cpu()), bits(scale.cpu()))
+    whole = (m // 32) * (k // 64) * 1536
+    assert torch.equal(tiles[:whole], quest.int4_to_e2m3_tiles(packed)[:whole])
+    del tiles
     step = 32768
     for lo in range(0, m, step):                      # in pieces: the unpacked codes of everything would be 2 GiB more
         codes = unpack_gpu(packed[lo:lo + step])
