@@ -269,6 +269,16 @@ int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_tiles, const v
                                        void *stream);
 
 /*
+ * quest_fused_matmul_dequantize_e2m3 adding its result to what mat_d holds: mat_d <- dtype(mat_d + dtype(product)), the two
+ * roundings of the framework's `x = x + linear(...)` (the residual additions of src/models/llama.py:175-176 with the
+ * projection that ends the branch, in one launch: the residual stream is read and written once and the branch's output
+ * never exists).  Every element of mat_d is read and written by the same lane; same shapes and limits.
+ */
+int quest_fused_matmul_dequantize_add_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles, const void *vec_a_mul,
+                                           const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
+                                           void *stream);
+
+/*
  * Diagnostic (host only, nothing is launched): how quest_fused_matmul_dequantize_e2m3 divides a shape among the
  * workgroups of a device with `cus` compute units.  plan[0..7] = workgroups, scheduling groups (one per XCD when 8),
  * tiles per token tile when every workgroup gets exactly one (else 0), how many ways the groups divide the token tiles

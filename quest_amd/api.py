@@ -401,12 +401,16 @@ def fused_matmul_dequantize_e2m3(
         size_k: int,
         out: torch.Tensor = None,
         swiglu: bool = False,
+        add_to_out: bool = False,
 ) -> torch.Tensor:
     """`fused_matmul_dequantize_int4_int4t_bf16` for codes held as E2M3 tiles: (M, N) outputs identical bit for bit,
     from the FP6 matrix instructions; the add vectors are not needed (2 C + a_add + b_add is twice the FP6 sum).
     M and N are the lengths of the scale vectors.  swiglu=True: the epilogue of
-    `fused_matmul_dequantize_swiglu_int4_int4t`, b in its interleaved row order, (M, N / 2) outputs."""
+    `fused_matmul_dequantize_swiglu_int4_int4t`, b in its interleaved row order, (M, N / 2) outputs.
+    add_to_out=True: `out` (required) becomes dtype(out + dtype(product)), the bits of `out + product` in torch -- the
+    residual addition after a projection, in the projection's launch."""
     m, n = vec_a_mul.numel(), vec_b_mul.numel()
+    assert not (add_to_out and (swiglu or out is None))
     if out is None:
         out = torch.empty(m, n // 2 if swiglu else n, dtype=vec_a_mul.dtype, device=a_tiles.device)
     assert a_tiles.dtype == torch.uint8 and b_tiles.dtype == torch.uint8 and a_tiles.is_contiguous() and b_tiles.is_contiguous()
@@ -416,6 +420,8 @@ def fused_matmul_dequantize_e2m3(
     assert out.shape == (m, n // 2 if swiglu else n)
     dev = require_gpu(a_tiles, b_tiles, vec_a_mul, vec_b_mul, out)
     fn = _lib.load().quest_fused_matmul_dequantize_swiglu_e2m3 if swiglu else _lib.load().quest_fused_matmul_dequantize_e2m3
+    if add_to_out:
+        fn = _lib.load().quest_fused_matmul_dequantize_add_e2m3
     with torch.cuda.device(dev):
         check(fn(ptr(out), ptr(a_tiles), ptr(b_tiles), ptr(vec_a_mul), ptr(vec_b_mul), m, size_k, n,
                  DTYPE_CODE[out.dtype], stream_of(out)), 'fused_matmul_dequantize_e2m3')

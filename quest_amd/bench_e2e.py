@@ -14,7 +14,8 @@ reference takes it):
   int4_had        W4A4 linears with the Hadamard transform, torch glue        (reference: int4 + HT)
   noop            no-op linears (they still rotate their input), torch glue   (reference: noop)
   fused           int4_had with the producer-fused blocks: norm / residual / SwiGLU inside the quantisers, rotary kernel
-  fused_noop      the same blocks with the GEMMs returning zeros: what of `fused` is not GEMM time
+  fused_noop      the same blocks with the GEMMs returning zeros (an output projection that would add into the residual
+                  stream leaves it untouched): what of `fused` is not GEMM time
 
     python -m quest_amd.bench_e2e [--model 1600m|213m] [--batch-sizes 1 2 4 8] [--matrix-path fp6|int8] [--json F] [--markdown F]
 
@@ -138,7 +139,10 @@ def main():
     ap.add_argument('--json', help='write the records to this file')
     ap.add_argument('--markdown', help='write the table to this file')
     ap.add_argument('--min-k', type=int, default=None, help='shortest rows that take the FP6 path (default: harness.E2M3_MIN_K)')
+    ap.add_argument('--no-gemm-add', action='store_true', help='residual additions in the norm kernels instead of the output projections\' GEMMs')
     args = ap.parse_args()
+    if args.no_gemm_add:
+        harness.GEMM_ADDS_RESIDUAL = False
     if args.min_k is not None:
         harness.E2M3_MIN_K = args.min_k
     if args.matrix_path is not None:

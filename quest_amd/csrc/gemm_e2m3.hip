@@ -160,10 +160,17 @@ __device__ __forceinline__ void k_step(v16f (&acc)[NA > 0 ? NA : 1][4], const Fr
     }
 }
 
-template <int OUT, bool GLU, int NA>
+// EPI: what the epilogue does with the scaled product -- kEpiPlain: store it; kEpiGlu: the gated unit over interleaved
+// weight rows; kEpiAdd: add it to what the output holds (the residual stream: dtype(out + dtype(product)), the two roundings
+// of the framework's x + linear(...), src/models/llama.py:175-176 of the reference).
+enum { kEpiPlain = 0, kEpiGlu = 1, kEpiAdd = 2 };
+
+template <int OUT, int EPI, int NA>
 __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, int M, int N, int K,
                                      int tok0, int ch0, int unit0, int width) {
     constexpr int DT = OUT;
+    constexpr bool GLU = EPI == kEpiGlu;
+    constexpr bool ADD = EPI == kEpiAdd;
     constexpr int NAX = NA > 0 ? NA : 1;
     const int wave = ldr.wave;                                      // scalar
     const int nk = K / 64;
@@ -261,8 +268,25 @@ __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe
                             ((size_t)(tok0 + tok_e + li_e) * n_out + (size_t)((ch0 >> 5) + unit0) * kOutPerUnit) * 2;
         auto convert_and_store = [&](auto guarded_tag) {
             constexpr bool kGuard = decltype(guarded_tag)::value;
+            // kEpiAdd: what the output holds under this lane's sixteen-byte pieces, fetched one channel unit ahead of
+            // the arithmetic that needs it (eight pieces per unit)
+            uint4 res[2][8];
+            auto fetch_unit = [&](int a, int par) {
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++) {
+                        const bool ok = !kGuard || (tok0 + tok_e + b * 32 + li_e < M && ch0 + (unit0 + a) * 32 + (2 * pr + lg_e) * 8 < N);
+                        res[par][b * 2 + pr] = make_uint4(0, 0, 0, 0);
+                        if (ok) res[par][b * 2 + pr] = *reinterpret_cast<const uint4 *>(out_lane + ((size_t)b * 32 * n_out + a * kOutPerUnit) * 2 + (2 * pr + lg_e) * 16);
+                    }
+            };
+            if constexpr (ADD) fetch_unit(0, 0);
 #pragma unroll
             for (int a = 0; a < NA; a++) {
+                if constexpr (ADD) {
+                    if (a + 1 < NA) fetch_unit(a + 1, (a + 1) & 1);
+                }
                 float muls[16];
 #pragma unroll
                 for (int rg = 0; rg < 4; rg++) {
@@ -301,7 +325,15 @@ __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe
                                 *reinterpret_cast<uint2 *>(dst + (2 * pr + lg_e) * 8) =
                                     make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
                         } else if (!kGuard || (tok_ok && ch0 + cl < N)) {
-                            *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                            uint4 o = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                            if constexpr (ADD) {
+                                const uint4 r = res[a & 1][b * 2 + pr];
+                                auto add2 = [](uint32_t p, uint32_t q) {
+                                    return pack2_rounded_products<DT>(__fadd_rn(lo_f32<DT>(q), lo_f32<DT>(p)), __fadd_rn(hi_f32<DT>(q), hi_f32<DT>(p)));
+                                };
+                                o = make_uint4(add2(o.x, r.x), add2(o.y, r.y), add2(o.z, r.z), add2(o.w, r.w));
+                            }
+                            *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = o;
                         }
                     }
                 }
@@ -323,7 +355,14 @@ __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe
                     if (ch0 + cl >= N) continue;
                     const float s = acc[a][b][r];
                     const float rhs = __fmul_rn(t_half_mul, to_f32<DT>(c_mul[cl]));
-                    reinterpret_cast<uint16_t *>(out)[(size_t)tok * N + ch0 + cl] = (uint16_t)from_f32<DT>(__fmul_rn(__fadd_rn(s, s), rhs));
+                    uint16_t *dst = reinterpret_cast<uint16_t *>(out) + (size_t)tok * N + ch0 + cl;
+                    uint32_t o = from_f32<DT>(__fmul_rn(__fadd_rn(s, s), rhs));
+                    if constexpr (ADD) {
+                        float sum = __fadd_rn(to_f32<DT>(*dst), to_f32<DT>((uint16_t)o));
+                        asm volatile("" : "+v"(sum));
+                        o = from_f32<DT>(sum);
+                    }
+                    *dst = (uint16_t)o;
                 }
         }
     }
@@ -334,7 +373,7 @@ __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe
     pp.vec_par ^= 1;
 }
 
-template <int OUT, bool GLU>
+template <int OUT, int EPI>
 __global__ void __launch_bounds__(256, 1)
 gemm_e2m3_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                  const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul, int M, int N, int K, Schedule sch) {
@@ -378,7 +417,7 @@ gemm_e2m3_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const 
         const int h0 = (cc.width + 1) >> 1;
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
-#define QUEST_E2M3_TILE(NA) tile<OUT, GLU, NA>(lds, ld, ldr, pp, out, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
+#define QUEST_E2M3_TILE(NA) tile<OUT, EPI, NA>(lds, ld, ldr, pp, out, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
         switch (na) {
             case 4: QUEST_E2M3_TILE(4); break;
             case 3: QUEST_E2M3_TILE(3); break;
@@ -430,16 +469,16 @@ __global__ void __launch_bounds__(256) int4_to_e2m3_tiles_kernel(uint8_t *__rest
 
 }  // namespace e2m3
 
-template <bool GLU>
+template <int EPI>
 static int launch_e2m3(int dtype, void *out, const uint8_t *a, const uint8_t *b, const void *a_mul, const void *b_mul, int M,
                        int K, int N, int cus, hipStream_t st) {
     long grid = 0;
     const Schedule sch = make_schedule(M, N, e2m3::kMaxUnits, 1, cus, &grid, e2m3::kTokSplit);
     if (dtype == QUEST_DTYPE_BF16)
-        e2m3::gemm_e2m3_kernel<OUT_BF16, GLU><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        e2m3::gemm_e2m3_kernel<OUT_BF16, EPI><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
             out, a, b, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
     else
-        e2m3::gemm_e2m3_kernel<OUT_FP16, GLU><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        e2m3::gemm_e2m3_kernel<OUT_FP16, EPI><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
             out, a, b, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
     return launch_status();
 }
@@ -486,8 +525,18 @@ extern "C" int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_til
     forget_stale_error();
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
-    return launch_e2m3<false>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+    return launch_e2m3<e2m3::kEpiPlain>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                               size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
+}
+
+extern "C" int quest_fused_matmul_dequantize_add_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles, const void *vec_a_mul,
+                                                      const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
+                                                      void *stream) {
+    forget_stale_error();
+    const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
+    if (rc != QUEST_OK) return rc;
+    return launch_e2m3<e2m3::kEpiAdd>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+                                      size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
 }
 
 extern "C" int quest_e2m3_gemm_plan(int size_m, int size_k, int size_n, int cus, int *plan) {
@@ -507,6 +556,6 @@ extern "C" int quest_fused_matmul_dequantize_swiglu_e2m3(void *mat_d, const void
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
     if (size_n & 7) return QUEST_ERR_BAD_SHAPE;
-    return launch_e2m3<true>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+    return launch_e2m3<e2m3::kEpiGlu>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                              size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
 }

@@ -23,6 +23,9 @@ WEIGHT_HADAMARD_SCALE = 2. ** -3.5      # utils.py:39
 MATRIX_PATH = 'fp6'
 E2M3_MIN_TILES = 66                     # 256 x 256 output tiles from which the FP6 kernel is the faster one
 E2M3_MIN_K = 2048                       # shortest rows that take it (see prefers_e2m3)
+# Whether a producer-fused block lets the FP6 GEMM of an output projection add into the residual stream itself
+# (same bits as the addition inside the next norm kernel; one pass over the stream less).
+GEMM_ADDS_RESIDUAL = True
 
 
 def prefers_e2m3(m: int, k: int, n: int) -> bool:
@@ -257,11 +260,18 @@ class Linear4bit(nn.Module):
             y += self.bias
         return y
 
-    def forward_tiles(self, a_scale, a_tiles, out=None) -> torch.Tensor:
-        """The same for activations quantised to E2M3 tiles: the GEMM on the FP6 matrix instructions."""
+    def forward_tiles(self, a_scale, a_tiles, out=None, add_to_out=False) -> torch.Tensor:
+        """The same for activations quantised to E2M3 tiles: the GEMM on the FP6 matrix instructions.  add_to_out: the
+        result is added to `out` (the residual stream) inside the GEMM's launch, with the bits of `out + layer(x)`."""
         if self.use_noop:
-            return self._noop_output(a_scale)
-        y = quest.fused_matmul_dequantize_e2m3(a_tiles, self.w_tiles(), a_scale, self.w_scale, self.weight.size(1), out)
+            return out if add_to_out else self._noop_output(a_scale)
+        if add_to_out and self.bias is not None:                     # out + (product + bias): the bias first, as torch would
+            y = quest.fused_matmul_dequantize_e2m3(a_tiles, self.w_tiles(), a_scale, self.w_scale, self.weight.size(1))
+            y += self.bias
+            out += y
+            return out
+        y = quest.fused_matmul_dequantize_e2m3(a_tiles, self.w_tiles(), a_scale, self.w_scale, self.weight.size(1), out,
+                                               add_to_out=add_to_out)
         if self.bias is not None:
             y += self.bias
         return y

@@ -155,6 +155,10 @@ class LlamaAttention(nn.Module):
 
     def attend(self, qkv, freqs_cis):
         """Everything after the QKV projection: qkv (B, T, 3 d) -> (B, T, d)."""
+        return self.c_proj(self.attention_core(qkv, freqs_cis))
+
+    def attention_core(self, qkv, freqs_cis):
+        """Rotary embedding and causal attention: qkv (B, T, 3 d) -> the input of the output projection (B, T, d)."""
         b, t, c3 = qkv.size()
         c = c3 // 3
         if self.fused_rope and qkv.is_cuda and qkv.is_contiguous():
@@ -162,7 +166,7 @@ class LlamaAttention(nn.Module):
             quest.rope_interleaved_(qkv, freqs_cis.contiguous(), 2 * c, c // self.n_head)
             q, k, v = (z.view(b, t, self.n_head, c // self.n_head).transpose(1, 2) for z in qkv.split(self.n_embd, dim=2))
             y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=True)
-            return self.c_proj(y.transpose(1, 2).contiguous().view(b, t, c))
+            return y.transpose(1, 2).contiguous().view(b, t, c)
         q, k, v = qkv.split(self.n_embd, dim=2)
         k = k.view(b, t, self.n_head, c // self.n_head)
         q = q.view(b, t, self.n_head, c // self.n_head)
@@ -170,7 +174,7 @@ class LlamaAttention(nn.Module):
         q, k = q.transpose(1, 2), k.transpose(1, 2)
         v = v.view(b, t, self.n_head, c // self.n_head).transpose(1, 2)
         y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=True)
-        return self.c_proj(y.transpose(1, 2).contiguous().view(b, t, c))
+        return y.transpose(1, 2).contiguous().view(b, t, c)
 
 
 class LlamaBlock(nn.Module):
@@ -188,7 +192,7 @@ class LlamaBlock(nn.Module):
     def forward(self, x, freqs_cis):
         if self.fuse_producers:
             x, branch = self.forward_fused(x, freqs_cis)
-            return x + branch
+            return x if branch is None else x + branch
         x = x + self.attn(self.ln_1(x), freqs_cis)
         return x + self.mlp(self.ln_2(x))
 
@@ -197,8 +201,9 @@ class LlamaBlock(nn.Module):
         c_attn and for the fused gate/up projection, silu(gate) * up -> codes for the MLP's c_proj.  Three bf16
         tensors per block (two normalised activations, one SwiGLU product) are never written or re-read, and the
         residual additions run inside the norm kernels: x is the residual stream, updated IN PLACE; `branch`, if
-        given, is the previous block's MLP output still to be added to it.  Returns (x, this block's MLP output):
-        the caller adds the last one (or hands it to the next block)."""
+        given, is the previous block's MLP output still to be added to it.  Returns (x, this block's MLP output or
+        None): the caller adds the last one (or hands it to the next block); None when the output projection's GEMM has
+        added it already."""
         b, t, c = x.shape
         m = b * t
         x2 = x.view(m, c)
@@ -217,10 +222,26 @@ class LlamaBlock(nn.Module):
             else:
                 q = quest.add_rmsnorm_hadamard_quantize_int4(x2, branch.view(m, c), self.ln_1.weight, self.ln_1.eps)
             qkv = self.attn.c_attn.forward_quantized(*q)
-        att = self.attn.attend(qkv.view(b, t, 3 * c), freqs_cis)
+        # the attention's output projection: on the FP6 path its GEMM adds into the residual stream itself (the bits of
+        # x + c_proj(...)) and the second norm has no addition left to do; otherwise the norm kernel adds
+        att = None
+        gemm_adds = harness.GEMM_ADDS_RESIDUAL
+        if gemm_adds and harness.prefers_e2m3(m, c, c) and isinstance(self.attn.c_proj, harness.Linear4bit) and self.attn.c_proj.use_hadamard:
+            core = self.attn.attention_core(qkv.view(b, t, 3 * c), freqs_cis)
+            self.attn.c_proj.forward_tiles(*quest.hadamard_quantize_e2m3(core.view(m, c)), out=x2, add_to_out=True)
+        else:
+            att = self.attn.attend(qkv.view(b, t, 3 * c), freqs_cis)
         down_tiles = harness.prefers_e2m3(m, hidden, c)
+
+        def second_norm(tiles: bool):
+            if att is None:
+                f = quest.rmsnorm_hadamard_quantize_e2m3 if tiles else quest.rmsnorm_hadamard_quantize_int4
+                return f(x2, self.ln_2.weight, self.ln_2.eps)
+            f = quest.add_rmsnorm_hadamard_quantize_e2m3 if tiles else quest.add_rmsnorm_hadamard_quantize_int4
+            return f(x2, att.view(m, c), self.ln_2.weight, self.ln_2.eps)
+
         if harness.prefers_e2m3(m, c, 2 * hidden):
-            q = quest.add_rmsnorm_hadamard_quantize_e2m3(x2, att.view(m, c), self.ln_2.weight, self.ln_2.eps)
+            q = second_norm(True)
             if self.mlp.glu is not None:
                 act = self.mlp.swiglu_tiles(*q)
                 q = quest.hadamard_quantize_e2m3(act) if down_tiles else quest.hadamard_quantize_int4(act)
@@ -228,13 +249,17 @@ class LlamaBlock(nn.Module):
                 gate_up = self.mlp.w12.forward_tiles(*q)
                 q = quest.silu_mul_hadamard_quantize_e2m3(gate_up) if down_tiles else quest.silu_mul_hadamard_quantize_int4(gate_up)
         else:
-            q = quest.add_rmsnorm_hadamard_quantize_int4(x2, att.view(m, c), self.ln_2.weight, self.ln_2.eps)
+            q = second_norm(False)
             if self.mlp.glu is not None:
                 act = self.mlp.swiglu_quantized(*q)
                 q = quest.hadamard_quantize_e2m3(act) if down_tiles else quest.hadamard_quantize_int4(act)
             else:
                 gate_up = self.mlp.w12.forward_quantized(*q)
                 q = quest.silu_mul_hadamard_quantize_e2m3(gate_up) if down_tiles else quest.silu_mul_hadamard_quantize_int4(gate_up)
+        if down_tiles and gemm_adds:
+            # the MLP's output projection adds into the residual stream as well: nothing is left for the caller to add
+            self.mlp.c_proj.forward_tiles(*q, out=x2, add_to_out=True)
+            return x, None
         y = self.mlp.c_proj.forward_tiles(*q) if down_tiles else self.mlp.c_proj.forward_quantized(*q)
         return x, y.view(b, t, c)
 

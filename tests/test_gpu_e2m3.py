@@ -161,6 +161,30 @@ def test_gemm_swiglu_equals_int8_kernel(quest, dtype, shape):
     assert torch.equal(bits(got.cpu()), bits(want.cpu()))
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(300, 256, 1000), (4096, 128, 4104), (1000, 512, 2048), (130, 384, 77), (2048, 2560, 2560), (33, 128, 8)])
+def test_gemm_adds_into_the_residual_stream(quest, dtype, shape):
+    """add_to_out: out <- dtype(out + dtype(product)), the bits of torch's `out + product` (interior and edge tiles, a
+    channel count that is not a multiple of 8, large and tiny residuals, twice in a row on the same buffer)."""
+    m, k, n = shape
+    g = torch.Generator(device=DEV).manual_seed(41)
+    a = torch.randint(0, 256, (m, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    b = torch.randint(0, 256, (n, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    a_mul = (torch.rand(m, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    ta, tb = quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(b)
+    product = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k)
+    res = (torch.randn(m, n, generator=g, device=DEV) * torch.rand(m, 1, generator=g, device=DEV) * 50).to(dtype)
+    res[0] *= 1e-4
+    want = res + product
+    got = res.clone()
+    ret = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k, out=got, add_to_out=True)
+    assert ret.data_ptr() == got.data_ptr()
+    assert torch.equal(bits(got.cpu()), bits(want.cpu()))
+    quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k, out=got, add_to_out=True)
+    assert torch.equal(bits(got.cpu()), bits((want + product).cpu()))
+
+
 def test_error_codes(quest):
     from quest_amd import _lib
     import ctypes
