@@ -279,6 +279,18 @@ int quest_fused_matmul_dequantize_add_e2m3(void *mat_d, const void *a_tiles, con
                                            void *stream);
 
 /*
+ * quest_fused_matmul_dequantize_e2m3 with quest_rope_interleaved applied to the first rot_cols channels of its result before
+ * it is stored (the q and k of a fused QKV projection, src/models/llama.py:134-140 with apply_rotary_emb, 43-62, in the
+ * projection's launch): row r is position r % seq_len of its sequence, the channels are heads of head_dim, pair i of a head
+ * turns by freqs_cis[r % seq_len][i] = (cos, sin) (fp32, (seq_len, head_dim / 2, 2), 16-byte aligned).  Bit for bit the
+ * two separate calls.  Limits beyond the plain entry point's: size_n % 8 == 0, head_dim % 32 == 0, rot_cols % head_dim == 0
+ * and <= size_n, seq_len >= 32 (QUEST_ERR_BAD_SHAPE otherwise -- make the two calls).
+ */
+int quest_fused_matmul_dequantize_rope_e2m3(void *mat_d, const void *a_tiles, const void *b_tiles, const void *vec_a_mul,
+                                            const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
+                                            const float *freqs_cis, int seq_len, int rot_cols, int head_dim, void *stream);
+
+/*
  * Diagnostic (host only, nothing is launched): how quest_fused_matmul_dequantize_e2m3 divides a shape among the
  * workgroups of a device with `cus` compute units.  plan[0..7] = workgroups, scheduling groups (one per XCD when 8),
  * tiles per token tile when every workgroup gets exactly one (else 0), how many ways the groups divide the token tiles

@@ -27,6 +27,7 @@ from .api import (  # noqa: F401
     e2m3_tiles_bytes,
     int4_to_e2m3_tiles,
     fused_matmul_dequantize_e2m3,
+    rope_gemm_fuses,
     hadamard_quantize_e2m3,
     rmsnorm_hadamard_quantize_e2m3,
     add_rmsnorm_hadamard_quantize_e2m3,

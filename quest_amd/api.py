@@ -393,6 +393,11 @@ def int4_to_e2m3_tiles(x_int_packed: torch.Tensor, out: torch.Tensor = None) -> 
     return out
 
 
+def rope_gemm_fuses(seq_len: int, n: int, rot_cols: int, head_dim: int) -> bool:
+    """Whether `fused_matmul_dequantize_e2m3(rope=...)` takes these shapes (otherwise: the GEMM, then `rope_interleaved_`)."""
+    return seq_len >= 32 and n % 8 == 0 and head_dim % 32 == 0 and 0 < rot_cols <= n and rot_cols % head_dim == 0
+
+
 def fused_matmul_dequantize_e2m3(
         a_tiles: torch.Tensor,
         b_tiles: torch.Tensor,
@@ -402,15 +407,19 @@ def fused_matmul_dequantize_e2m3(
         out: torch.Tensor = None,
         swiglu: bool = False,
         add_to_out: bool = False,
+        rope: tuple = None,
 ) -> torch.Tensor:
     """`fused_matmul_dequantize_int4_int4t_bf16` for codes held as E2M3 tiles: (M, N) outputs identical bit for bit,
     from the FP6 matrix instructions; the add vectors are not needed (2 C + a_add + b_add is twice the FP6 sum).
     M and N are the lengths of the scale vectors.  swiglu=True: the epilogue of
     `fused_matmul_dequantize_swiglu_int4_int4t`, b in its interleaved row order, (M, N / 2) outputs.
     add_to_out=True: `out` (required) becomes dtype(out + dtype(product)), the bits of `out + product` in torch -- the
-    residual addition after a projection, in the projection's launch."""
+    residual addition after a projection, in the projection's launch.
+    rope=(freqs_cis, rot_cols, head_dim): `rope_interleaved_` on the first rot_cols channels of the result, in the same
+    launch and with the same bits; row r is position r % T of its sequence, T = freqs_cis.size(0) (see `rope_gemm_fuses`
+    for the shapes this takes)."""
     m, n = vec_a_mul.numel(), vec_b_mul.numel()
-    assert not (add_to_out and (swiglu or out is None))
+    assert not (add_to_out and (swiglu or out is None)) and not (rope is not None and (swiglu or add_to_out))
     if out is None:
         out = torch.empty(m, n // 2 if swiglu else n, dtype=vec_a_mul.dtype, device=a_tiles.device)
     assert a_tiles.dtype == torch.uint8 and b_tiles.dtype == torch.uint8 and a_tiles.is_contiguous() and b_tiles.is_contiguous()
@@ -422,6 +431,16 @@ def fused_matmul_dequantize_e2m3(
     fn = _lib.load().quest_fused_matmul_dequantize_swiglu_e2m3 if swiglu else _lib.load().quest_fused_matmul_dequantize_e2m3
     if add_to_out:
         fn = _lib.load().quest_fused_matmul_dequantize_add_e2m3
+    if rope is not None:
+        freqs_cis, rot_cols, head_dim = rope
+        assert freqs_cis.dtype == torch.float32 and freqs_cis.is_contiguous() and freqs_cis.shape[1:] == (head_dim // 2, 2)
+        assert rope_gemm_fuses(freqs_cis.size(0), n, rot_cols, head_dim), 'shape outside the fused rotary epilogue'
+        require_gpu(freqs_cis, out)
+        with torch.cuda.device(dev):
+            check(_lib.load().quest_fused_matmul_dequantize_rope_e2m3(
+                ptr(out), ptr(a_tiles), ptr(b_tiles), ptr(vec_a_mul), ptr(vec_b_mul), m, size_k, n, DTYPE_CODE[out.dtype],
+                ptr(freqs_cis), freqs_cis.size(0), rot_cols, head_dim, stream_of(out)), 'fused_matmul_dequantize_rope_e2m3')
+        return out
     with torch.cuda.device(dev):
         check(fn(ptr(out), ptr(a_tiles), ptr(b_tiles), ptr(vec_a_mul), ptr(vec_b_mul), m, size_k, n,
                  DTYPE_CODE[out.dtype], stream_of(out)), 'fused_matmul_dequantize_e2m3')

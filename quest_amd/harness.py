@@ -26,6 +26,8 @@ E2M3_MIN_K = 2048                       # shortest rows that take it (see prefer
 # Whether a producer-fused block lets the FP6 GEMM of an output projection add into the residual stream itself
 # (same bits as the addition inside the next norm kernel; one pass over the stream less).
 GEMM_ADDS_RESIDUAL = True
+# ... and the rotary embedding of q and k after the fused QKV projection (the FP6 GEMM's rotary epilogue)
+GEMM_ROTATES_QK = True
 
 
 def prefers_e2m3(m: int, k: int, n: int) -> bool:
@@ -260,9 +262,11 @@ class Linear4bit(nn.Module):
             y += self.bias
         return y
 
-    def forward_tiles(self, a_scale, a_tiles, out=None, add_to_out=False) -> torch.Tensor:
+    def forward_tiles(self, a_scale, a_tiles, out=None, add_to_out=False, rope=None) -> torch.Tensor:
         """The same for activations quantised to E2M3 tiles: the GEMM on the FP6 matrix instructions.  add_to_out: the
-        result is added to `out` (the residual stream) inside the GEMM's launch, with the bits of `out + layer(x)`."""
+        result is added to `out` (the residual stream) inside the GEMM's launch, with the bits of `out + layer(x)`.
+        rope = (freqs_cis, rot_cols, head_dim): the rotary embedding of the first rot_cols channels in the GEMM's launch
+        (layers without a bias; the caller checks `quest.rope_gemm_fuses`)."""
         if self.use_noop:
             return out if add_to_out else self._noop_output(a_scale)
         if add_to_out and self.bias is not None:                     # out + (product + bias): the bias first, as torch would
@@ -270,8 +274,9 @@ class Linear4bit(nn.Module):
             y += self.bias
             out += y
             return out
+        assert rope is None or self.bias is None
         y = quest.fused_matmul_dequantize_e2m3(a_tiles, self.w_tiles(), a_scale, self.w_scale, self.weight.size(1), out,
-                                               add_to_out=add_to_out)
+                                               add_to_out=add_to_out, rope=rope)
         if self.bias is not None:
             y += self.bias
         return y

@@ -153,17 +153,19 @@ class LlamaAttention(nn.Module):
     def forward(self, x, freqs_cis):
         return self.attend(self.c_attn(x), freqs_cis)
 
-    def attend(self, qkv, freqs_cis):
+    def attend(self, qkv, freqs_cis, rotated=False):
         """Everything after the QKV projection: qkv (B, T, 3 d) -> (B, T, d)."""
-        return self.c_proj(self.attention_core(qkv, freqs_cis))
+        return self.c_proj(self.attention_core(qkv, freqs_cis, rotated))
 
-    def attention_core(self, qkv, freqs_cis):
-        """Rotary embedding and causal attention: qkv (B, T, 3 d) -> the input of the output projection (B, T, d)."""
+    def attention_core(self, qkv, freqs_cis, rotated=False):
+        """Rotary embedding (unless the projection has `rotated` q and k already) and causal attention: qkv (B, T, 3 d)
+        -> the input of the output projection (B, T, d)."""
         b, t, c3 = qkv.size()
         c = c3 // 3
-        if self.fused_rope and qkv.is_cuda and qkv.is_contiguous():
+        if (rotated or self.fused_rope) and qkv.is_cuda and qkv.is_contiguous():
             # q and k rotated where they lie in the projection's output (one kernel, bit-identical to apply_rotary_emb)
-            quest.rope_interleaved_(qkv, freqs_cis.contiguous(), 2 * c, c // self.n_head)
+            if not rotated:
+                quest.rope_interleaved_(qkv, freqs_cis.contiguous(), 2 * c, c // self.n_head)
             q, k, v = (z.view(b, t, self.n_head, c // self.n_head).transpose(1, 2) for z in qkv.split(self.n_embd, dim=2))
             y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=True)
             return y.transpose(1, 2).contiguous().view(b, t, c)
@@ -210,12 +212,21 @@ class LlamaBlock(nn.Module):
         hidden = self.mlp.c_proj.weight.size(1)
         # each producer writes the operand form its GEMM runs fastest on: E2M3 tiles for the FP6 kernel, or packed
         # nibbles and row sums for the INT8 kernels (same codes, same output bits either way)
+        rotated = False
         if harness.prefers_e2m3(m, c, 3 * c):
             if branch is None:
                 q = quest.rmsnorm_hadamard_quantize_e2m3(x2, self.ln_1.weight, self.ln_1.eps)
             else:
                 q = quest.add_rmsnorm_hadamard_quantize_e2m3(x2, branch.view(m, c), self.ln_1.weight, self.ln_1.eps)
-            qkv = self.attn.c_attn.forward_tiles(*q)
+            # ... whose GEMM also rotates q and k where the shapes allow (the bits of the separate rotary kernel)
+            head_dim = c // self.attn.n_head
+            c_attn = self.attn.c_attn
+            if (harness.GEMM_ROTATES_QK and self.attn.fused_rope and isinstance(c_attn, harness.Linear4bit)
+                    and c_attn.bias is None and not c_attn.use_noop and quest.rope_gemm_fuses(t, 3 * c, 2 * c, head_dim)):
+                qkv = c_attn.forward_tiles(*q, rope=(freqs_cis.contiguous(), 2 * c, head_dim))
+                rotated = True
+            else:
+                qkv = c_attn.forward_tiles(*q)
         else:
             if branch is None:
                 q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
@@ -227,10 +238,10 @@ class LlamaBlock(nn.Module):
         att = None
         gemm_adds = harness.GEMM_ADDS_RESIDUAL
         if gemm_adds and harness.prefers_e2m3(m, c, c) and isinstance(self.attn.c_proj, harness.Linear4bit) and self.attn.c_proj.use_hadamard:
-            core = self.attn.attention_core(qkv.view(b, t, 3 * c), freqs_cis)
+            core = self.attn.attention_core(qkv.view(b, t, 3 * c), freqs_cis, rotated)
             self.attn.c_proj.forward_tiles(*quest.hadamard_quantize_e2m3(core.view(m, c)), out=x2, add_to_out=True)
         else:
-            att = self.attn.attend(qkv.view(b, t, 3 * c), freqs_cis)
+            att = self.attn.attend(qkv.view(b, t, 3 * c), freqs_cis, rotated)
         down_tiles = harness.prefers_e2m3(m, hidden, c)
 
         def second_norm(tiles: bool):

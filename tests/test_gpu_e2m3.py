@@ -185,6 +185,51 @@ def test_gemm_adds_into_the_residual_stream(quest, dtype, shape):
     assert torch.equal(bits(got.cpu()), bits((want + product).cpu()))
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [
+    # batch, sequence, K, heads, head_dim, extra channels after q, k, v
+    (2, 150, 256, 3, 32, 0), (1, 4096, 128, 2, 64, 0), (3, 100, 512, 5, 96, 0), (2, 512, 2560, 20, 128, 0),
+    (5, 33, 128, 1, 128, 8), (1, 32, 128, 2, 32, 0)])
+def test_gemm_rotates_q_and_k(quest, dtype, shape):
+    """rope=...: the GEMM's output with the first 2 d channels rotated = the plain GEMM followed by the rotary kernel, bit
+    for bit (positions wrapping at every sequence, heads narrower and wider than a tile's channel unit, edge tiles, a
+    trailing block of channels that is not a head)."""
+    bsz, t, k, heads, hd, extra = shape
+    m, c = bsz * t, heads * hd
+    n = 3 * c + extra
+    g = torch.Generator(device=DEV).manual_seed(43)
+    a = torch.randint(0, 256, (m, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    b = torch.randint(0, 256, (n, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    a_mul = (torch.rand(m, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    ang = torch.rand(t, hd // 2, generator=g, device=DEV) * 6.283
+    freqs = torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).contiguous()
+    ta, tb = quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(b)
+    want = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k)
+    plain = want.clone()
+    quest.rope_interleaved_(want.view(bsz, t, n), freqs, 2 * c, hd)
+    assert quest.rope_gemm_fuses(t, n, 2 * c, hd)
+    got = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k, rope=(freqs, 2 * c, hd))
+    assert torch.equal(bits(got.cpu()), bits(want.cpu()))
+    assert torch.equal(bits(got[:, 2 * c:].cpu()), bits(plain[:, 2 * c:].cpu()))           # v (and what follows) untouched
+    assert not torch.equal(bits(got[:, :2 * c].cpu()), bits(plain[:, :2 * c].cpu()))
+
+
+def test_rope_epilogue_rejects_what_it_does_not_take(quest):
+    from quest_amd import _lib
+    import ctypes
+    lib = _lib.load()
+    null, fake = ctypes.c_void_p(0), ctypes.c_void_p(0x1000)
+    call = lambda n, seq, rot, hd, f=fake: lib.quest_fused_matmul_dequantize_rope_e2m3(fake, fake, fake, fake, fake, 64, 128, n, 0, f, seq, rot, hd, null)
+    assert call(384, 64, 256, 128, null) == -1
+    assert call(384, 16, 256, 128) == -2          # sequences shorter than 32
+    assert call(384, 64, 256, 48) == -2           # heads that are not whole 32-channel units
+    assert call(384, 64, 200, 128) == -2          # rotated channels that are not whole heads
+    assert call(384, 64, 512, 128) == -2          # ... or more than there are
+    assert call(386, 64, 256, 128) == -2          # channel count not a multiple of 8
+    assert not quest.rope_gemm_fuses(16, 384, 256, 128) and not quest.rope_gemm_fuses(64, 384, 256, 48)
+
+
 def test_error_codes(quest):
     from quest_amd import _lib
     import ctypes
