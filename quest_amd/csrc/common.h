@@ -315,6 +315,16 @@ inline int aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t
 // earlier call left behind (a failed call of the caller's in this thread, a failed device query in here) is read and
 // dropped first: forget_stale_error() before the first launch of an entry point, launch_status() after the last.
 inline void forget_stale_error() { (void)hipGetLastError(); }
+
+// Compute units of the device the stream belongs to.  Asked for once per call that needs it (two host-side queries,
+// no stream operation, nothing cached): the library keeps no state and a process may drive several devices.
+inline int device_cu_count(hipStream_t st) {
+    int dev = 0, cus = 0;
+    const bool found = hipStreamGetDevice(st, &dev) == hipSuccess || hipGetDevice(&dev) == hipSuccess;
+    const bool counted = found && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0;
+    forget_stale_error();                      // a failed query must not be taken for the launch that follows
+    return counted ? cus : 256;
+}
 inline int launch_status() { return hipGetLastError() == hipSuccess ? QUEST_OK : QUEST_ERR_LAUNCH; }
 
 }  // namespace quest

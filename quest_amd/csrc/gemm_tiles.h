@@ -41,16 +41,6 @@ __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
     }
 }
 
-// Compute units of the device the stream belongs to.  Asked for once per call that needs it (two host-side queries,
-// no stream operation, nothing cached): the library keeps no state and a process may drive several devices.
-inline int device_cu_count(hipStream_t st) {
-    int dev = 0, cus = 0;
-    const bool found = hipStreamGetDevice(st, &dev) == hipSuccess || hipGetDevice(&dev) == hipSuccess;
-    const bool counted = found && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0;
-    forget_stale_error();                      // a failed query must not be taken for the launch that follows
-    return counted ? cus : 256;
-}
-
 // gemm_big.hip: the large-tile kernel (K % 128 == 0, 4-byte aligned scale vectors); `duo` picks two workgroups of
 // 256 x 128 tiles per CU instead of one of 256 x 256, `glu` the SwiGLU epilogue (16-bit outputs only), `cus` the
 // device's CU count (the persistent grid's size)

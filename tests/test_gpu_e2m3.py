@@ -251,10 +251,13 @@ def rand_act(m, k, dtype, seed):
 
 
 ACT_SHAPES = [(64, 4096), (33, 1024), (70, 128), (5, 2816), (1, 4096), (257, 256), (40, 11008), (9, 8192), (130, 512), (3, 32768)]
+# enough rows for workgroups of eight (four) whole rows that stage the tiles in LDS (at least two per compute unit), with a
+# ragged last workgroup: rows of one wave's blocks, of fewer, and of two and three waves
+STAGED_SHAPES = [(4101, 2560), (4099, 1024), (2051, 6912), (2050, 11008)]
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
-@pytest.mark.parametrize('shape', ACT_SHAPES)
+@pytest.mark.parametrize('shape', ACT_SHAPES + STAGED_SHAPES)
 def test_activation_tiles_hold_the_packed_codes(quest, dtype, shape):
     """The tiles written by the fused activation kernel decode to exactly the codes its packed output holds (which the
     parity tests pin against the oracle), with the same scale, in one launch and in a launch that writes tiles only."""
@@ -289,7 +292,7 @@ def test_activation_tiles_degenerate_rows(quest, dtype):
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
-@pytest.mark.parametrize('shape', [(64, 4096), (33, 1024), (70, 128), (5, 2816), (40, 11008), (130, 512), (3, 32768)])
+@pytest.mark.parametrize('shape', [(64, 4096), (33, 1024), (70, 128), (5, 2816), (40, 11008), (130, 512), (3, 32768), (4101, 2560)])
 def test_no_transform_on_the_matrix_core_kernel(quest, dtype, shape):
     """hadamard_scale = 0 with rows of whole blocks of 128: the matrix-core kernel without its multiplications (the
     loaded chunks only change lanes).  The scale is the oracle's on x itself (one ulp: summation order), the codes are the
@@ -335,7 +338,7 @@ def test_tiles_fall_back_without_the_matrix_core_transform(quest, dtype):
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
-@pytest.mark.parametrize('shape', [(64, 1024), (33, 4096), (20, 6912), (9, 11008)])
+@pytest.mark.parametrize('shape', [(64, 1024), (33, 4096), (20, 6912), (9, 11008), (4100, 1024), (2052, 6912)])
 def test_producer_kernels_write_the_same_tiles(quest, dtype, shape):
     m, k = shape
     g = torch.Generator().manual_seed(24)
