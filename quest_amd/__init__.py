@@ -28,6 +28,7 @@ from .api import (  # noqa: F401
     int4_to_e2m3_tiles,
     fused_matmul_dequantize_e2m3,
     rope_gemm_fuses,
+    fused_matmul_dequantize_rope_int4_int4t,
     hadamard_quantize_e2m3,
     rmsnorm_hadamard_quantize_e2m3,
     add_rmsnorm_hadamard_quantize_e2m3,

@@ -55,6 +55,44 @@ def fused_matmul_dequantize_int4_int4t_bf16(
     return out
 
 
+def fused_matmul_dequantize_rope_int4_int4t(
+        mat_a: torch.Tensor,
+        mat_b: torch.Tensor,
+        vec_a_add: torch.Tensor,
+        vec_b_add: torch.Tensor,
+        vec_a_mul: torch.Tensor,
+        vec_b_mul: torch.Tensor,
+        freqs_cis: torch.Tensor,
+        rot_cols: int,
+        head_dim: int,
+        out: torch.Tensor = None,
+) -> torch.Tensor:
+    """`fused_matmul_dequantize_int4_int4t_bf16` followed by `rope_interleaved_` on the first rot_cols channels (row r is
+    position r % T of its sequence, T = freqs_cis.size(0)): in the GEMM's launch where the large-tile kernel takes the
+    shape, as the two calls otherwise -- the same bits either way."""
+    m, n, t = mat_a.size(0), mat_b.size(0), freqs_cis.size(0)
+    if out is None:
+        out = torch.empty(m, n, dtype=vec_a_mul.dtype, device=mat_a.device)
+    assert mat_a.dtype == torch.uint8 and mat_b.dtype == torch.uint8 and vec_a_add.dtype == torch.int32 and vec_b_add.dtype == torch.int32
+    assert vec_a_mul.dtype in _FLOAT16S and vec_b_mul.dtype == vec_a_mul.dtype and out.dtype == vec_a_mul.dtype
+    assert mat_a.is_contiguous() and mat_b.is_contiguous() and vec_a_add.is_contiguous() and vec_b_add.is_contiguous() and vec_a_mul.is_contiguous() and vec_b_mul.is_contiguous() and out.is_contiguous()
+    assert mat_a.size(1) == mat_b.size(1) and vec_a_add.numel() == m and vec_a_mul.numel() == m
+    assert vec_b_add.numel() == n and vec_b_mul.numel() == n and out.shape == (m, n)
+    assert freqs_cis.dtype == torch.float32 and freqs_cis.is_contiguous() and freqs_cis.shape == (t, head_dim // 2, 2)
+    assert m % t == 0 and 0 < rot_cols <= n and rot_cols % head_dim == 0
+    dev = require_gpu(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, freqs_cis, out)
+    with torch.cuda.device(dev):
+        rc = _lib.load().quest_fused_matmul_dequantize_rope_int4_int4t(
+            ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
+            m, mat_b.size(1) * 2, n, DTYPE_CODE[out.dtype], ptr(freqs_cis), t, rot_cols, head_dim, stream_of(out))
+    if rc in (QUEST_ERR_UNSUPPORTED, QUEST_ERR_BAD_SHAPE):          # nothing was launched: the two calls
+        fused_matmul_dequantize_int4_int4t_bf16(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, out)
+        rope_interleaved_(out.view(m // t, t, n), freqs_cis, rot_cols, head_dim)
+        return out
+    check(rc, 'fused_matmul_dequantize_rope_int4_int4t')
+    return out
+
+
 GEMM_WORKSPACE_MAX_BYTES = 16384 + (2 << 20)         # the most quest_gemm_workspace_bytes returns for any shape
 
 

@@ -62,8 +62,9 @@ static int small_tile_shape(int M, int K, int N, int cus) {
 // faster shape, and within 7 % on every single size.
 static int gemm_launch_large(int out_kind, bool glu, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                              const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus,
-                             hipStream_t st) {
+                             hipStream_t st, const RopeArgs *rope = nullptr) {
     const int small_shape = small_tile_shape(M, K, N, cus);
+    if (small_shape != 0 && rope != nullptr) return QUEST_ERR_UNSUPPORTED;        // the small tiles have no rotary epilogue
     if (small_shape != 0) return launch_gemm_small(out_kind, glu, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     const int units = (N + 31) / 32;
     const int per_group = units >= 8 ? units / 8 : units;
@@ -71,7 +72,8 @@ static int gemm_launch_large(int out_kind, bool glu, void *out, const uint8_t *a
     // small problems (fewer cells per group than Wide has workgroups): twice the workgroups help while K is short
     const bool small = cells_per_group <= 32 && K <= (cells_per_group <= 24 ? 4096 : 2816);
     const bool duo = small || (cells_per_group >= 256 && (K <= 1024 || per_group <= 16));
-    return launch_gemm_big(out_kind, glu, duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
+    return launch_gemm_big(out_kind, rope != nullptr ? kEpiRope : glu ? kEpiGlu : kEpiPlain, duo, out, a, b, a_add, b_add, a_mul, b_mul,
+                           M, K, N, cus, st, rope);
 }
 
 static int gemm_launch(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
@@ -197,6 +199,29 @@ extern "C" int quest_fused_matmul_dequantize_int4_int4t_noalloc(void *mat_d, con
     if (split != QUEST_ERR_UNSUPPORTED) return split;
     return gemm_launch(out_kind, mat_d, mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, size_m, size_k, size_n,
                        (hipStream_t)stream);
+}
+
+extern "C" int quest_fused_matmul_dequantize_rope_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                             const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                             const void *vec_a_mul, const void *vec_b_mul, int size_m,
+                                                             int size_k, int size_n, int dtype, const float *freqs_cis,
+                                                             int seq_len, int rot_cols, int head_dim, void *stream) {
+    forget_stale_error();
+    const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
+    if (rc != QUEST_OK) return rc;
+    if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul || !freqs_cis) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    if (seq_len < 32 || rot_cols <= 0 || head_dim <= 0 || (head_dim & 31) || (rot_cols % head_dim) || rot_cols > size_n || (size_n & 7))
+        return QUEST_ERR_BAD_SHAPE;
+    if (!aligned(freqs_cis, 16)) return QUEST_ERR_ALIGNMENT;
+    // only the large-tile kernel has this epilogue (the same sizes the plain entry point hands to it)
+    if ((size_k & 127) != 0 || size_m <= 64 || (size_m <= 128 && size_n <= 8192) || !aligned(vec_b_mul, 4) || !aligned(vec_a_mul, 4) ||
+        !aligned(mat_d, 16))
+        return QUEST_ERR_UNSUPPORTED;
+    const RopeArgs rope = {freqs_cis, seq_len, rot_cols, head_dim};
+    return gemm_launch_large(dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16, false, mat_d, mat_a, mat_b, vec_a_add, vec_b_add,
+                             vec_a_mul, vec_b_mul, size_m, size_k, size_n, device_cu_count((hipStream_t)stream),
+                             (hipStream_t)stream, &rope);
 }
 
 extern "C" int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,

@@ -176,12 +176,15 @@ __device__ __forceinline__ void k_pair(v16i (&acc)[NA > 0 ? NA : 1][4], const Fr
     }
 }
 
-template <typename C, int OUT, bool GLU, int NA, int TB>
+template <typename C, int OUT, int EPI, int NA, int TB>
 __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, const int32_t *__restrict__ a_add,
                                          const int32_t *__restrict__ b_add, const uint16_t *__restrict__ a_mul,
                                          const uint16_t *__restrict__ b_mul, int M, int N, int K, int tok0, int ch0,
-                                         int unit0, int width) {
+                                         int unit0, int width, const RopeArgs &rope) {
     constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
+    constexpr bool GLU = EPI == kEpiGlu;
+    constexpr bool ROPE = EPI == kEpiRope;
+    static_assert(EPI == kEpiPlain || OUT != OUT_INT32, "epilogues on 16-bit outputs only");
     constexpr int NAX = NA > 0 ? NA : 1;
     // Lane coordinates are derived afresh in every phase (here, in the loader's cursor step, in the epilogue): a value
     // computed once from threadIdx would be kept alive across the whole kernel, spilled to scratch at the register
@@ -352,10 +355,20 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
         // interior tiles (the common case) store without the per-lane bounds tests and their exec-mask branches
         auto convert_and_store = [&](auto guarded_tag) {
         constexpr bool kGuard = decltype(guarded_tag)::value;
+        // kEpiRope: the angles of this lane's sixteen-byte pieces, fetched one piece ahead in the order of the loops below
+        constexpr int kOuter = kTokOuter ? TB : NA, kInner = kTokOuter ? NA : TB;
+        float4 cs[2][2];
+        RopeLane rl = {0, 0};
+        if constexpr (ROPE) rl = rope_lane(rope, tok0 + tok_e + li_e, ch0 + unit0 * 32);
+        auto fetch_angles = [&](int piece, int par) {
+            const int o = piece / (2 * kInner), i = (piece >> 1) % kInner;
+            rope_fetch(rope, rl, lg_e, kTokOuter ? i : o, kTokOuter ? o : i, piece & 1, cs[par]);
+        };
+        if constexpr (ROPE) fetch_angles(0, 0);
 #pragma unroll
-        for (int o = 0; o < (kTokOuter ? TB : NA); o++) {
+        for (int o = 0; o < kOuter; o++) {
 #pragma unroll
-          for (int i = 0; i < (kTokOuter ? NA : TB); i++) {
+          for (int i = 0; i < kInner; i++) {
             const int a = kTokOuter ? i : o, b = kTokOuter ? o : i;
             if constexpr (OUT != OUT_INT32 && !kTokOuter) {
               if (i == 0) load_scales(a, adds_u[0], muls_u[0]);
@@ -395,6 +408,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                         const auto s0 = __builtin_amdgcn_permlane32_swap(x[2 * pr][0], x[2 * pr + 1][0], false, false);
                         const auto s1 = __builtin_amdgcn_permlane32_swap(x[2 * pr][1], x[2 * pr + 1][1], false, false);
                         const int cl = (unit0 + a) * 32 + (2 * pr + lg_e) * 8;
+                        if constexpr (ROPE) {
+                            constexpr int kPieces = 2 * kOuter * kInner;
+                            const int nxt = (o * kInner + i) * 2 + pr + 1;
+                            if (nxt < kPieces) fetch_angles(nxt, (pr + 1) & 1);
+                        }
                         if constexpr (GLU) {
                             // The weight rows come interleaved in eights, four gate rows then the four up rows of the same
                             // outputs: after the swap a lane holds exactly such an eight, gates in (s0[0], s1[0]), ups in
@@ -403,7 +421,11 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                                 *reinterpret_cast<uint2 *>(dst + (2 * pr + lg_e) * 8) =
                                     make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
                         } else if (!kGuard || (tok_ok && ch0 + cl < N)) {
-                            *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                            uint4 piece = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                            if constexpr (ROPE) {
+                                if (ch0 + cl < rope.rot_cols) piece = rope_turn<DT>(piece, cs[pr]);
+                            }
+                            *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = piece;
                         }
                     }
                 }
@@ -460,12 +482,12 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     pp.vec_par ^= 1;
 }
 
-template <typename C, int OUT, bool GLU>
+template <typename C, int OUT, int EPI>
 __global__ void __launch_bounds__(256, C::kWgPerCu)
 gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                      const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
                      const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
-                     int M, int N, int K, Schedule sch) {
+                     int M, int N, int K, Schedule sch, RopeArgs rope) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[C::kLdsB];
     // wave-uniform by construction; readfirstlane tells the compiler so, which keeps everything that is
     // updated under `switch (na)` below (cursors, slot numbers, LDS bases) in scalar registers; the empty
@@ -515,14 +537,14 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
         const int na = wc == 0 ? h0 : cc.width - h0;
         const int unit0 = wc == 0 ? 0 : h0;
 #define QUEST_BIG_TILE(NA) \
-    big_tile<C, OUT, GLU, NA, 4>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width)
+    big_tile<C, OUT, EPI, NA, 4>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, unit0, cc.width, rope)
         if (cc.width <= 2) {
             // a tile of one or two channel units (small problems, the ends of runs): every wave takes a quarter of the
             // tokens and all of the units, instead of two of the four waves idling or holding half-empty accumulators
             if (cc.width == 2)
-                big_tile<C, OUT, GLU, 2, 2>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, 0, 2);
+                big_tile<C, OUT, EPI, 2, 2>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, 0, 2, rope);
             else
-                big_tile<C, OUT, GLU, 1, 2>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, 0, 1);
+                big_tile<C, OUT, EPI, 1, 2>(lds, ld, ldr, pp, out, a_add, b_add, a_mul, b_mul, M, N, K, cc.tok0, cc.ch0, 0, 1, rope);
         } else if constexpr (C::kMaxUnits > 4) {
             switch (na) {
                 case 4: QUEST_BIG_TILE(4); break;
@@ -546,35 +568,38 @@ gemm_w4a4_big_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, co
 
 }  // namespace big
 
-template <typename C, int OUT, bool GLU>
+template <typename C, int OUT, int EPI>
 static int launch_big(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                           const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
+                           const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st, const RopeArgs &rope) {
     long grid = 0;
     const Schedule sch = make_schedule(M, N, C::kMaxUnits, C::kWgPerCu, cus, &grid);
-    big::gemm_w4a4_big_kernel<C, OUT, GLU><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
-        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch);
+    big::gemm_w4a4_big_kernel<C, OUT, EPI><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, sch, rope);
     return launch_status();
 }
 
-template <int OUT, bool GLU>
+template <int OUT, int EPI>
 static int launch_shape(bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                        const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
-    if (duo) return launch_big<big::Duo, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
-    return launch_big<big::Wide, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
+                        const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st, const RopeArgs &rope) {
+    if (duo) return launch_big<big::Duo, OUT, EPI>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope);
+    return launch_big<big::Wide, OUT, EPI>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope);
 }
 
-int launch_gemm_big(int out_kind, bool glu, bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
-                    const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st) {
-    if ((K & 127) != 0 || cus <= 0 || (glu && out_kind == OUT_INT32)) return QUEST_ERR_UNSUPPORTED;
-    if (glu) {
-        if (out_kind == OUT_BF16) return launch_shape<OUT_BF16, true>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
-        return launch_shape<OUT_FP16, true>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
-    }
-    switch (out_kind) {
-        case OUT_BF16: return launch_shape<OUT_BF16, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
-        case OUT_FP16: return launch_shape<OUT_FP16, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
-        default: return launch_shape<OUT_INT32, false>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st);
-    }
+int launch_gemm_big(int out_kind, int epi, bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                    const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st,
+                    const RopeArgs *rope_args) {
+    if ((K & 127) != 0 || cus <= 0 || (epi != kEpiPlain && out_kind == OUT_INT32)) return QUEST_ERR_UNSUPPORTED;
+    if (epi == kEpiRope && rope_args == nullptr) return QUEST_ERR_NULL_POINTER;
+    const RopeArgs rope = epi == kEpiRope ? *rope_args : RopeArgs{nullptr, 32, 0, 32};
+#define QUEST_BIG_EPI(E)                                                                                                            \
+    (out_kind == OUT_BF16 ? launch_shape<OUT_BF16, E>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope)            \
+                          : launch_shape<OUT_FP16, E>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope))
+    if (epi == kEpiGlu) return QUEST_BIG_EPI(kEpiGlu);
+    if (epi == kEpiRope) return QUEST_BIG_EPI(kEpiRope);
+    if (epi != kEpiPlain) return QUEST_ERR_UNSUPPORTED;
+    if (out_kind == OUT_INT32) return launch_shape<OUT_INT32, kEpiPlain>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope);
+    return QUEST_BIG_EPI(kEpiPlain);
+#undef QUEST_BIG_EPI
 }
 
 }  // namespace quest

@@ -160,20 +160,6 @@ __device__ __forceinline__ void k_step(v16f (&acc)[NA > 0 ? NA : 1][4], const Fr
     }
 }
 
-// EPI: what the epilogue does with the scaled product -- kEpiPlain: store it; kEpiGlu: the gated unit over interleaved
-// weight rows; kEpiAdd: add it to what the output holds (the residual stream: dtype(out + dtype(product)), the two roundings
-// of the framework's x + linear(...), src/models/llama.py:175-176 of the reference).
-enum { kEpiPlain = 0, kEpiGlu = 1, kEpiAdd = 2, kEpiRope = 3 };
-
-// kEpiRope: the rotary embedding of the reference (src/models/llama.py:43-62) on the first rot_cols channels of the output
-// -- q and k of a fused QKV projection -- applied to the rounded product before it is stored: channels are heads of
-// head_dim, a head is (re, im) pairs, pair i of a head at position t = row % seq_len turns by freqs[t][i] = (cos, sin);
-// fp32 products and sums in the reference's order, one more rounding to dtype.  The arithmetic of rope_kernel (rowops.hip).
-struct RopeArgs {
-    const float *freqs;
-    int seq_len, rot_cols, head_dim;
-};
-
 template <int OUT, int EPI, int NA>
 __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe &pp, void *__restrict__ out, int M, int N, int K,
                                      int tok0, int ch0, int unit0, int width, const RopeArgs &rope) {
@@ -292,33 +278,12 @@ __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe
                     }
             };
             if constexpr (ADD) fetch_unit(0, 0);
-            // kEpiRope: (cos, sin) of the four pairs in this lane's sixteen-byte piece, fetched one piece ahead (pieces in
-            // the order of the loops below: unit a, token block b, half pr).  Byte offsets into the table: the lane's first
-            // token row's position in its sequence (row % seq_len, one division per tile; the other three blocks are 32, 64
-            // and 96 rows on, seq_len >= 32) and its column inside a 32-channel unit; a unit lies inside one head
-            // (head_dim is a multiple of 32), whose first channel's place in the head is wave-uniform.
+            // kEpiRope: the angles of this lane's sixteen-byte pieces, fetched one piece ahead (pieces in the order of the
+            // loops below: unit a, token block b, half pr)
             float4 cs[2][2];
-            int t_first = 0, head_at = 0;
-            if constexpr (ROPE) {
-                // the divisor through an opaque copy: the reciprocal is then worked out here, once per tile, instead of
-                // living in a vector register (or in scratch memory) across the whole tile loop
-                int seq_len = rope.seq_len;
-                asm volatile("" : "+s"(seq_len));
-                t_first = (tok0 + tok_e + li_e) % seq_len;
-                head_at = __builtin_amdgcn_readfirstlane((ch0 + unit0 * 32) % rope.head_dim);
-            }
-            auto fetch_angles = [&](int piece, int par) {
-                const int a = piece >> 3, b = (piece >> 1) & 3, pr = piece & 1;
-                int h = head_at + a * 32;                          // a < 8 and head_dim >= 32: at most 8 wraps, uniform
-                while (h >= rope.head_dim) h -= rope.head_dim;
-                int t = t_first + b * 32;
-#pragma unroll
-                for (int i = 0; i < 3; i++) t = t >= rope.seq_len ? t - rope.seq_len : t;
-                const uint8_t *f = reinterpret_cast<const uint8_t *>(rope.freqs) +
-                                   ((uint32_t)t * (uint32_t)rope.head_dim * 4u + lg_e * 32u) + (h * 4 + pr * 64);
-                cs[par][0] = *reinterpret_cast<const float4 *>(f);
-                cs[par][1] = *reinterpret_cast<const float4 *>(f + 16);
-            };
+            RopeLane rl = {0, 0};
+            if constexpr (ROPE) rl = rope_lane(rope, tok0 + tok_e + li_e, ch0 + unit0 * 32);
+            auto fetch_angles = [&](int piece, int par) { rope_fetch(rope, rl, lg_e, piece >> 3, (piece >> 1) & 3, piece & 1, cs[par]); };
             if constexpr (ROPE) fetch_angles(0, 0);
 #pragma unroll
             for (int a = 0; a < NA; a++) {
@@ -368,16 +333,7 @@ __device__ __forceinline__ void tile(uint8_t *lds, Cursor &ld, Loader &ldr, Pipe
                         } else if (!kGuard || (tok_ok && ch0 + cl < N)) {
                             uint4 o = make_uint4(s0[0], s1[0], s0[1], s1[1]);
                             if constexpr (ROPE) {
-                                if (ch0 + cl < rope.rot_cols) {
-                                    const float4 f01 = cs[pr][0], f23 = cs[pr][1];
-                                    auto turn = [](uint32_t p, float c, float sn) {
-                                        const float re = lo_f32<DT>(p), im = hi_f32<DT>(p);
-                                        float out_re = __fsub_rn(__fmul_rn(re, c), __fmul_rn(im, sn));
-                                        float out_im = __fadd_rn(__fmul_rn(re, sn), __fmul_rn(im, c));
-                                        return pack2_rounded_products<DT>(out_re, out_im);
-                                    };
-                                    o = make_uint4(turn(o.x, f01.x, f01.y), turn(o.y, f01.z, f01.w), turn(o.z, f23.x, f23.y), turn(o.w, f23.z, f23.w));
-                                }
+                                if (ch0 + cl < rope.rot_cols) o = rope_turn<DT>(o, cs[pr]);
                             }
                             if constexpr (ADD) {
                                 const uint4 r = res[a & 1][b * 2 + pr];
@@ -525,7 +481,7 @@ __global__ void __launch_bounds__(256) int4_to_e2m3_tiles_kernel(uint8_t *__rest
 
 template <int EPI>
 static int launch_e2m3(int dtype, void *out, const uint8_t *a, const uint8_t *b, const void *a_mul, const void *b_mul, int M,
-                       int K, int N, int cus, hipStream_t st, e2m3::RopeArgs rope = e2m3::RopeArgs{nullptr, 1, 0, 2}) {
+                       int K, int N, int cus, hipStream_t st, RopeArgs rope = RopeArgs{nullptr, 1, 0, 2}) {
     long grid = 0;
     const Schedule sch = make_schedule(M, N, e2m3::kMaxUnits, 1, cus, &grid, e2m3::kTokSplit);
     if (dtype == QUEST_DTYPE_BF16)
@@ -579,7 +535,7 @@ extern "C" int quest_fused_matmul_dequantize_e2m3(void *mat_d, const void *a_til
     forget_stale_error();
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
-    return launch_e2m3<e2m3::kEpiPlain>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+    return launch_e2m3<kEpiPlain>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                               size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
 }
 
@@ -589,7 +545,7 @@ extern "C" int quest_fused_matmul_dequantize_add_e2m3(void *mat_d, const void *a
     forget_stale_error();
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
-    return launch_e2m3<e2m3::kEpiAdd>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+    return launch_e2m3<kEpiAdd>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                                       size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
 }
 
@@ -604,9 +560,9 @@ extern "C" int quest_fused_matmul_dequantize_rope_e2m3(void *mat_d, const void *
     if (seq_len < 32 || rot_cols <= 0 || head_dim <= 0 || (head_dim & 31) || (rot_cols % head_dim) || rot_cols > size_n || (size_n & 7))
         return QUEST_ERR_BAD_SHAPE;
     if (!aligned(freqs_cis, 16)) return QUEST_ERR_ALIGNMENT;
-    return launch_e2m3<e2m3::kEpiRope>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+    return launch_e2m3<kEpiRope>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                                        size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream,
-                                       e2m3::RopeArgs{freqs_cis, seq_len, rot_cols, head_dim});
+                                       RopeArgs{freqs_cis, seq_len, rot_cols, head_dim});
 }
 
 extern "C" int quest_e2m3_gemm_plan(int size_m, int size_k, int size_n, int cus, int *plan) {
@@ -626,6 +582,6 @@ extern "C" int quest_fused_matmul_dequantize_swiglu_e2m3(void *mat_d, const void
     const int rc = e2m3_gemm_check(mat_d, a_tiles, b_tiles, vec_a_mul, vec_b_mul, size_m, size_k, size_n, dtype);
     if (rc != QUEST_OK) return rc;
     if (size_n & 7) return QUEST_ERR_BAD_SHAPE;
-    return launch_e2m3<e2m3::kEpiGlu>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
+    return launch_e2m3<kEpiGlu>(dtype, mat_d, (const uint8_t *)a_tiles, (const uint8_t *)b_tiles, vec_a_mul, vec_b_mul, size_m,
                              size_k, size_n, device_cu_count((hipStream_t)stream), (hipStream_t)stream);
 }

@@ -243,12 +243,17 @@ class Linear4bit(nn.Module):
         self.bias = nn.Parameter(torch.zeros(out_features, dtype=dtype, device=device), requires_grad=False) if bias else None
         return self
 
-    def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None) -> torch.Tensor:
+    def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None, rope=None) -> torch.Tensor:
         """The GEMM half of `linear_forward` on activations some fused producer kernel has already quantised:
         (M, 1) scales, (M, K/2) codes, (M, 1) row sums -> (M, N).  In no-op mode the GEMM is skipped (zeros), which is
-        what prices the GEMMs of a producer-fused model: everything else, the quantising producers included, still runs."""
+        what prices the GEMMs of a producer-fused model: everything else, the quantising producers included, still runs.
+        rope = (freqs_cis, rot_cols, head_dim): the first rot_cols channels leave rotated (layers without a bias)."""
         if self.use_noop:
             return self._noop_output(a_scale)
+        if rope is not None:
+            assert self.bias is None
+            return quest.fused_matmul_dequantize_rope_int4_int4t(a_int_packed, self.w_int_packed, a_int_row_sum, self.w_add,
+                                                                 a_scale, self.w_scale, *rope, out=out)
         y = quest.fused_matmul_dequantize_int4_int4t_bf16(mat_a=a_int_packed, mat_b=self.w_int_packed,
                                                           vec_a_add=a_int_row_sum, vec_b_add=self.w_add,
                                                           vec_a_mul=a_scale, vec_b_mul=self.w_scale, out=out)

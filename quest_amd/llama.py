@@ -232,7 +232,14 @@ class LlamaBlock(nn.Module):
                 q = quest.rmsnorm_hadamard_quantize_int4(x2, self.ln_1.weight, self.ln_1.eps)
             else:
                 q = quest.add_rmsnorm_hadamard_quantize_int4(x2, branch.view(m, c), self.ln_1.weight, self.ln_1.eps)
-            qkv = self.attn.c_attn.forward_quantized(*q)
+            c_attn = self.attn.c_attn
+            if (harness.GEMM_ROTATES_QK and self.attn.fused_rope and isinstance(c_attn, harness.Linear4bit)
+                    and c_attn.bias is None and not c_attn.use_noop and m % t == 0):
+                # (in the GEMM's launch where the large-tile kernel takes the shape, as a second launch otherwise)
+                qkv = c_attn.forward_quantized(*q, rope=(freqs_cis.contiguous(), 2 * c, c // self.attn.n_head))
+                rotated = True
+            else:
+                qkv = c_attn.forward_quantized(*q)
         # the attention's output projection: on the FP6 path its GEMM adds into the residual stream itself (the bits of
         # x + c_proj(...)) and the second norm has no addition left to do; otherwise the norm kernel adds
         att = None
