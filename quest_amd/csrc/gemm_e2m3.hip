@@ -56,12 +56,18 @@ struct Loader {          // direct-to-LDS loads of one wave: waves 0, 1 bring th
 
 __device__ __forceinline__ void loader_offsets(Loader &l, const Cursor &ld, int lane) {
     const int rb0 = ((l.wave < 2 ? ld.tok0 : ld.ch0) >> 5) + (l.wave & 1) * 4;
-    // row blocks past the matrix give offsets past the buffer: such loads touch no memory and return zeros
+    // row blocks past the matrix give offsets past the buffer: such loads touch no memory and return zeros.  So do the
+    // channel units past the tile's width (the tiles are smaller than 2 GiB): a narrow tile fetches what it multiplies,
+    // while every wave still issues the same number of loads per step.
+    const int units = l.wave < 2 ? 8 : ld.width;             // row blocks of this side the tile uses
+    const int first = (l.wave & 1) * 4;
 #pragma unroll
-    for (int j = 0; j < 4; j++) l.off[j] = (uint32_t)(rb0 + j) * (uint32_t)l.pitch + lane * 16;
+    for (int j = 0; j < 4; j++)
+        l.off[j] = first + j < units ? (uint32_t)(rb0 + j) * (uint32_t)l.pitch + lane * 16 : 0x80000000u;
 #pragma unroll
     for (int j = 0; j < 2; j++)
-        l.off[4 + j] = (uint32_t)(rb0 + 2 * j + (lane >> 5)) * (uint32_t)l.pitch + kHeadB + (lane & 31) * 16;
+        l.off[4 + j] = first + 2 * j + (lane >> 5) < units
+                           ? (uint32_t)(rb0 + 2 * j + (lane >> 5)) * (uint32_t)l.pitch + kHeadB + (lane & 31) * 16 : 0x80000000u;
 }
 
 // Load j of the cursor's step: the head of fragment 4 wave + j (j < 4), or the tails of fragments 4 wave + 2 (j - 4) and
