@@ -281,10 +281,10 @@ int quest_fused_matmul_dequantize_add_e2m3(void *mat_d, const void *a_tiles, con
 /*
  * quest_fused_matmul_dequantize_int4_int4t with quest_rope_interleaved applied to the first rot_cols channels of its result
  * before it is stored (`self.c_attn(x)` followed by `apply_rotary_emb(q, k, freqs_cis)`, src/models/llama.py:134-140 and
- * 43-62, in one launch), on packed codes: arguments and limits as quest_fused_matmul_dequantize_rope_e2m3 below.  Only the
- * large-tile kernel has this epilogue: QUEST_ERR_UNSUPPORTED (nothing launched) for the sizes the plain entry point gives to
- * another kernel (size_m <= 64, few small tiles, size_k % 128 != 0, scale vectors or output not 4- / 16-byte aligned) --
- * make the two calls then.
+ * 43-62, in one launch), on packed codes: arguments and limits as quest_fused_matmul_dequantize_rope_e2m3 below.  The
+ * large-tile and the small-tile kernels have this epilogue: QUEST_ERR_UNSUPPORTED (nothing launched) for the sizes the plain
+ * entry point gives to another kernel (size_m <= 64, size_m <= 128 with size_n <= 8192, size_k % 128 != 0, scale vectors or
+ * output not 4- / 16-byte aligned) -- make the two calls then.
  */
 int quest_fused_matmul_dequantize_rope_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
                                                   const int32_t *vec_a_add, const int32_t *vec_b_add, const void *vec_a_mul,

@@ -64,16 +64,15 @@ static int gemm_launch_large(int out_kind, bool glu, void *out, const uint8_t *a
                              const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus,
                              hipStream_t st, const RopeArgs *rope = nullptr) {
     const int small_shape = small_tile_shape(M, K, N, cus);
-    if (small_shape != 0 && rope != nullptr) return QUEST_ERR_UNSUPPORTED;        // the small tiles have no rotary epilogue
-    if (small_shape != 0) return launch_gemm_small(out_kind, glu, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    const int epi = rope != nullptr ? kEpiRope : glu ? kEpiGlu : kEpiPlain;
+    if (small_shape != 0) return launch_gemm_small(out_kind, epi, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope);
     const int units = (N + 31) / 32;
     const int per_group = units >= 8 ? units / 8 : units;
     const long cells_per_group = (long)((M + kBigTileRows - 1) / kBigTileRows) * per_group;
     // small problems (fewer cells per group than Wide has workgroups): twice the workgroups help while K is short
     const bool small = cells_per_group <= 32 && K <= (cells_per_group <= 24 ? 4096 : 2816);
     const bool duo = small || (cells_per_group >= 256 && (K <= 1024 || per_group <= 16));
-    return launch_gemm_big(out_kind, rope != nullptr ? kEpiRope : glu ? kEpiGlu : kEpiPlain, duo, out, a, b, a_add, b_add, a_mul, b_mul,
-                           M, K, N, cus, st, rope);
+    return launch_gemm_big(out_kind, epi, duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope);
 }
 
 static int gemm_launch(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
@@ -81,7 +80,7 @@ static int gemm_launch(int out_kind, void *out, const uint8_t *a, const uint8_t 
     // the device is asked for its CU count once per call, and only where a rule below uses it (not for a handful of tokens)
     const int cus = M > 64 ? device_cu_count(st) : 0;
     const int small_shape = small_tile_shape(M, K, N, cus);
-    if (small_shape != 0) return launch_gemm_small(out_kind, false, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+    if (small_shape != 0) return launch_gemm_small(out_kind, kEpiPlain, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
     // a handful of tokens: the weight-streaming kernel
     // (up to 64 of them unless the small tiles took the call above; where K rules those out, up to 128 while its
     // N / 16 workgroups still run as one round: twice as fast as large tiles that would be half empty)
@@ -214,7 +213,7 @@ extern "C" int quest_fused_matmul_dequantize_rope_int4_int4t(void *mat_d, const 
     if (seq_len < 32 || rot_cols <= 0 || head_dim <= 0 || (head_dim & 31) || (rot_cols % head_dim) || rot_cols > size_n || (size_n & 7))
         return QUEST_ERR_BAD_SHAPE;
     if (!aligned(freqs_cis, 16)) return QUEST_ERR_ALIGNMENT;
-    // only the large-tile kernel has this epilogue (the same sizes the plain entry point hands to it)
+    // the large-tile and the small-tile kernels have this epilogue (the sizes the plain entry point hands to them)
     if ((size_k & 127) != 0 || size_m <= 64 || (size_m <= 128 && size_n <= 8192) || !aligned(vec_b_mul, 4) || !aligned(vec_a_mul, 4) ||
         !aligned(mat_d, 16))
         return QUEST_ERR_UNSUPPORTED;

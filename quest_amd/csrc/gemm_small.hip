@@ -46,14 +46,17 @@ struct Shape {
 using Tile64 = Shape<1, 1, 4>;
 using Tile128 = Shape<2, 2, 2>;
 
-template <typename S, int OUT, bool GLU>
+template <typename S, int OUT, int EPI>
 __global__ void __launch_bounds__(512, 2 * S::kWgPerCu)
 gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, const uint8_t *__restrict__ wgt,
                        const int32_t *__restrict__ a_add, const int32_t *__restrict__ b_add,
                        const uint16_t *__restrict__ a_mul, const uint16_t *__restrict__ b_mul,
-                       int M, int N, int K, int tiles_t, int tiles_c) {
+                       int M, int N, int K, int tiles_t, int tiles_c, RopeArgs rope) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[S::kLdsB];
     constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
+    constexpr bool GLU = EPI == kEpiGlu;
+    constexpr bool ROPE = EPI == kEpiRope;            // (the caller guarantees N % 8 == 0 and a 16-byte aligned output)
+    static_assert(EPI == kEpiPlain || OUT != OUT_INT32, "epilogues on 16-bit outputs only");
     constexpr int NA = S::kUnits, TW = S::kTokWaves;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int lane = (int)threadIdx.x & 63;
@@ -224,7 +227,18 @@ gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, 
                         *reinterpret_cast<uint2 *>(dst + (c >> 1)) =
                             make_uint2(silu_mul_pair<DT>(s0[0], s0[1]), silu_mul_pair<DT>(s1[0], s1[1]));
                 } else if (tok_ok && c < N) {
-                    *reinterpret_cast<uint4 *>(dst + c) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                    uint4 piece8 = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                    if constexpr (ROPE) {
+                        // q and k of a fused QKV projection leave rotated: the piece's four (re, im) pairs by the angles of
+                        // its row's position in its sequence (the other waves of the CU cover the fetch)
+                        if (c < rope.rot_cols) {
+                            const int t = tok % rope.seq_len, h = c % rope.head_dim;
+                            const float4 *f = reinterpret_cast<const float4 *>(rope.freqs + ((size_t)t * (rope.head_dim >> 1) + (h >> 1)) * 2);
+                            const float4 cs[2] = {f[0], f[1]};
+                            piece8 = rope_turn<DT>(piece8, cs);
+                        }
+                    }
+                    *reinterpret_cast<uint4 *>(dst + c) = piece8;
                 }
             } else if (!GLU && tok_ok) {
 #pragma unroll
@@ -241,36 +255,39 @@ gemm_w4a4_small_kernel(void *__restrict__ out, const uint8_t *__restrict__ act, 
 
 }  // namespace small
 
-template <typename S, int OUT, bool GLU>
+template <typename S, int OUT, int EPI>
 static int launch_small(void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                             const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
+                             const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st, const RopeArgs &rope) {
     const int tiles_t = (M + S::kTok - 1) / S::kTok;
     const int tiles_c = (N + S::kChn - 1) / S::kChn;
     const long grid = (long)tiles_t * ((tiles_c + 7) / 8) * 8;
-    small::gemm_w4a4_small_kernel<S, OUT, GLU><<<dim3((unsigned)grid), dim3(512), 0, st>>>(
-        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, tiles_t, tiles_c);
+    small::gemm_w4a4_small_kernel<S, OUT, EPI><<<dim3((unsigned)grid), dim3(512), 0, st>>>(
+        out, a, b, a_add, b_add, (const uint16_t *)a_mul, (const uint16_t *)b_mul, M, N, K, tiles_t, tiles_c, rope);
     return launch_status();
 }
 
-template <int OUT, bool GLU>
+template <int OUT, int EPI>
 static int launch_shape(int shape, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add, const int32_t *b_add,
-                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    if (shape == 128) return launch_small<small::Tile128, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    return launch_small<small::Tile64, OUT, GLU>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
+                        const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st, const RopeArgs &rope) {
+    if (shape == 128) return launch_small<small::Tile128, OUT, EPI>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope);
+    return launch_small<small::Tile64, OUT, EPI>(out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope);
 }
 
-int launch_gemm_small(int out_kind, bool glu, int shape, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
-                      const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st) {
-    if ((K & 255) != 0 || (shape != 64 && shape != 128) || (glu && out_kind == OUT_INT32)) return QUEST_ERR_UNSUPPORTED;
-    if (glu) {
-        if (out_kind == OUT_BF16) return launch_shape<OUT_BF16, true>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        return launch_shape<OUT_FP16, true>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    }
-    switch (out_kind) {
-        case OUT_BF16: return launch_shape<OUT_BF16, false>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        case OUT_FP16: return launch_shape<OUT_FP16, false>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-        default: return launch_shape<OUT_INT32, false>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st);
-    }
+int launch_gemm_small(int out_kind, int epi, int shape, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                      const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st,
+                      const RopeArgs *rope_args) {
+    if ((K & 255) != 0 || (shape != 64 && shape != 128) || (epi != kEpiPlain && out_kind == OUT_INT32)) return QUEST_ERR_UNSUPPORTED;
+    if (epi == kEpiRope && (rope_args == nullptr || (N & 7) != 0 || !aligned(out, 16))) return QUEST_ERR_UNSUPPORTED;
+    const RopeArgs rope = epi == kEpiRope ? *rope_args : RopeArgs{nullptr, 32, 0, 32};
+#define QUEST_SMALL_EPI(E)                                                                                                   \
+    (out_kind == OUT_BF16 ? launch_shape<OUT_BF16, E>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope)        \
+                          : launch_shape<OUT_FP16, E>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope))
+    if (epi == kEpiGlu) return QUEST_SMALL_EPI(kEpiGlu);
+    if (epi == kEpiRope) return QUEST_SMALL_EPI(kEpiRope);
+    if (epi != kEpiPlain) return QUEST_ERR_UNSUPPORTED;
+    if (out_kind == OUT_INT32) return launch_shape<OUT_INT32, kEpiPlain>(shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope);
+    return QUEST_SMALL_EPI(kEpiPlain);
+#undef QUEST_SMALL_EPI
 }
 
 }  // namespace quest

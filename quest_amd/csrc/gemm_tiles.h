@@ -103,9 +103,10 @@ __device__ __forceinline__ void split16(const v4i &p, v4i &even, v4i &odd) {
 int launch_gemm_big(int out_kind, int epi, bool duo, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                     const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus, hipStream_t st,
                     const RopeArgs *rope = nullptr);
-// gemm_small.hip: tiles of `shape` x `shape` (64 or 128), K % 256 == 0
-int launch_gemm_small(int out_kind, bool glu, int shape, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
-                      const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);
+// gemm_small.hip: tiles of `shape` x `shape` (64 or 128), K % 256 == 0; `epi` as above
+int launch_gemm_small(int out_kind, int epi, int shape, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
+                      const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st,
+                      const RopeArgs *rope = nullptr);
 // gemm_staged.hip: K % 32 == 0, scale vectors at any element offset
 int launch_gemm_staged(int out_kind, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                        const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, hipStream_t st);

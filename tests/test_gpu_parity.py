@@ -274,16 +274,10 @@ def test_swiglu_gemm_refuses_small_batches(quest):
                                                         torch.ones(n, 1, dtype=torch.bfloat16, device=DEV))
 
 
-def _large_tile_kernel_takes(m, k, n):
-    """The dispatch of the fused GEMM (gemm.hip), restated: whether the large-tile kernel gets this size."""
-    if k % 128 or m <= 64 or (m <= 128 and n <= 8192):
-        return False
-    if k % 256 == 0:
-        cus = torch.cuda.get_device_properties(0).multi_processor_count
-        per_cu = -(-(-(-m // 64) * -(-n // 64)) // cus)
-        if per_cu <= 4 or (per_cu <= 8 and m < 1024 and m % 256):
-            return False
-    return True
+def _tiled_kernel_takes(m, k, n):
+    """The dispatch of the fused GEMM (gemm.hip), restated: whether the large-tile or the small-tile kernel gets this size
+    (the two with the rotary epilogue) rather than the weight-streaming or the register-staged one."""
+    return k % 128 == 0 and m > 64 and not (m <= 128 and n <= 8192)
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
@@ -291,12 +285,13 @@ def _large_tile_kernel_takes(m, k, n):
     # batch, sequence, K, heads, head_dim, channels after q and k
     (2, 150, 384, 3, 32, 96), (32, 512, 128, 8, 64, 0), (32, 512, 128, 4, 64, 256), (3, 100, 384, 5, 96, 480),
     (8, 512, 1024, 16, 64, 1024), (5, 33, 128, 1, 128, 136), (4, 64, 128, 1, 32, 0), (1, 48, 256, 2, 64, 128),
-    (2, 128, 256, 2, 32, 64), (2, 40, 160, 2, 32, 64)])
+    (2, 128, 256, 2, 32, 64), (2, 40, 160, 2, 32, 64), (1, 512, 2560, 20, 128, 2560), (3, 100, 512, 4, 64, 264),
+    (4, 512, 256, 16, 128, 2048)])
 def test_fused_matmul_dequantize_rope(quest, dtype, shape):
     """The QKV projection whose q and k leave the GEMM rotated = the plain fused GEMM followed by the rotary kernel, bit
-    for bit: both shapes of the large-tile kernel, tiles of one or two channel units, edge tiles, positions wrapping at
-    every sequence -- and the sizes that another kernel takes (a handful of tokens, few small tiles, K % 128 != 0), where
-    the call is the two launches."""
+    for bit: both shapes of the large-tile kernel, tiles of one or two channel units, both small-tile shapes, edge tiles,
+    positions wrapping at every sequence -- and the sizes that another kernel takes (a handful of tokens, K % 128 != 0),
+    where the call is the two launches."""
     bsz, t, k, heads, hd, rest = shape
     m, c = bsz * t, heads * hd
     n = 2 * c + rest
@@ -318,7 +313,7 @@ def test_fused_matmul_dequantize_rope(quest, dtype, shape):
     rc = _lib.load().quest_fused_matmul_dequantize_rope_int4_int4t(
         got.data_ptr(), a.data_ptr(), b.data_ptr(), a_add.data_ptr(), b_add.data_ptr(), a_mul.data_ptr(), b_mul.data_ptr(),
         m, k, n, 0 if dtype == torch.bfloat16 else 1, freqs.data_ptr(), t, 2 * c, hd, torch.cuda.current_stream().cuda_stream)
-    assert rc == (0 if _large_tile_kernel_takes(m, k, n) else -5), rc
+    assert rc == (0 if _tiled_kernel_takes(m, k, n) else -5), rc
     torch.cuda.synchronize()
 
 
