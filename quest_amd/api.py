@@ -68,7 +68,7 @@ def fused_matmul_dequantize_rope_int4_int4t(
         out: torch.Tensor = None,
 ) -> torch.Tensor:
     """`fused_matmul_dequantize_int4_int4t_bf16` followed by `rope_interleaved_` on the first rot_cols channels (row r is
-    position r % T of its sequence, T = freqs_cis.size(0)): in the GEMM's launch where the large-tile kernel takes the
+    position r % T of its sequence, T = freqs_cis.size(0)): in the GEMM's launch where a tiled kernel takes the
     shape, as the two calls otherwise -- the same bits either way."""
     m, n, t = mat_a.size(0), mat_b.size(0), freqs_cis.size(0)
     if out is None:

@@ -235,7 +235,7 @@ class LlamaBlock(nn.Module):
             c_attn = self.attn.c_attn
             if (harness.GEMM_ROTATES_QK and self.attn.fused_rope and isinstance(c_attn, harness.Linear4bit)
                     and c_attn.bias is None and not c_attn.use_noop and m % t == 0):
-                # (in the GEMM's launch where the large-tile kernel takes the shape, as a second launch otherwise)
+                # (in the GEMM's launch where a tiled kernel takes the shape, as a second launch for a handful of tokens)
                 qkv = c_attn.forward_quantized(*q, rope=(freqs_cis.contiguous(), 2 * c, c // self.attn.n_head))
                 rotated = True
             else:
