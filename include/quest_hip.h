@@ -279,6 +279,19 @@ int quest_fused_matmul_dequantize_add_e2m3(void *mat_d, const void *a_tiles, con
                                            void *stream);
 
 /*
+ * quest_fused_matmul_dequantize_int4_int4t adding its result to what mat_d holds: mat_d <- dtype(mat_d + dtype(product)), the
+ * two roundings of the framework's `x = x + linear(...)` (src/models/llama.py:175-176 with the projection that ends the
+ * branch, in one launch), on packed codes.  Only the large-tile kernel has this epilogue: QUEST_ERR_UNSUPPORTED (nothing
+ * launched) for the sizes the plain entry point gives to another kernel; quest_fused_matmul_dequantize_add_available says
+ * beforehand (1 / 0) whether a size runs in one launch on the stream's device.  mat_d 16-byte aligned.
+ */
+int quest_fused_matmul_dequantize_add_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                 const int32_t *vec_a_add, const int32_t *vec_b_add, const void *vec_a_mul,
+                                                 const void *vec_b_mul, int size_m, int size_k, int size_n, int dtype,
+                                                 void *stream);
+int quest_fused_matmul_dequantize_add_available(int size_m, int size_k, int size_n, void *stream);
+
+/*
  * quest_fused_matmul_dequantize_int4_int4t with quest_rope_interleaved applied to the first rot_cols channels of its result
  * before it is stored (`self.c_attn(x)` followed by `apply_rotary_emb(q, k, freqs_cis)`, src/models/llama.py:134-140 and
  * 43-62, in one launch), on packed codes: arguments and limits as quest_fused_matmul_dequantize_rope_e2m3 below.  The

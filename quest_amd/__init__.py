@@ -29,6 +29,8 @@ from .api import (  # noqa: F401
     fused_matmul_dequantize_e2m3,
     rope_gemm_fuses,
     fused_matmul_dequantize_rope_int4_int4t,
+    fused_matmul_dequantize_add_int4_int4t,
+    gemm_add_fuses,
     hadamard_quantize_e2m3,
     rmsnorm_hadamard_quantize_e2m3,
     add_rmsnorm_hadamard_quantize_e2m3,

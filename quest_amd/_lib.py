@@ -44,6 +44,8 @@ SIGNATURES = {
     'quest_int4_to_e2m3_tiles': [_vp, _vp, _i, _i, _vp],
     'quest_fused_matmul_dequantize_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     'quest_fused_matmul_dequantize_add_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    'quest_fused_matmul_dequantize_add_int4_int4t': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    'quest_fused_matmul_dequantize_add_available': [_i, _i, _i, _vp],
     'quest_fused_matmul_dequantize_rope_int4_int4t': [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp],
     'quest_fused_matmul_dequantize_rope_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp],
     'quest_fused_matmul_dequantize_swiglu_e2m3': [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],

@@ -8,6 +8,8 @@ kernels reached through the C ABI of libquest_hip.so.  Differences, all additive
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -90,6 +92,44 @@ def fused_matmul_dequantize_rope_int4_int4t(
         rope_interleaved_(out.view(m // t, t, n), freqs_cis, rot_cols, head_dim)
         return out
     check(rc, 'fused_matmul_dequantize_rope_int4_int4t')
+    return out
+
+
+def gemm_add_fuses(size_m: int, size_k: int, size_n: int, device=None) -> bool:
+    """Whether `fused_matmul_dequantize_add_int4_int4t` runs this size as one launch on `device` (the current one by default)."""
+    dev = torch.device('cuda', torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        return bool(_lib.load().quest_fused_matmul_dequantize_add_available(
+            size_m, size_k, size_n, ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)))
+
+
+def fused_matmul_dequantize_add_int4_int4t(
+        mat_a: torch.Tensor,
+        mat_b: torch.Tensor,
+        vec_a_add: torch.Tensor,
+        vec_b_add: torch.Tensor,
+        vec_a_mul: torch.Tensor,
+        vec_b_mul: torch.Tensor,
+        out: torch.Tensor,
+) -> torch.Tensor:
+    """out <- dtype(out + dtype(product)) with the product of `fused_matmul_dequantize_int4_int4t_bf16`: the bits of torch's
+    `out + product` (the residual addition after a projection), in the GEMM's launch where `gemm_add_fuses` says so and as
+    two launches otherwise."""
+    m, n = mat_a.size(0), mat_b.size(0)
+    assert mat_a.dtype == torch.uint8 and mat_b.dtype == torch.uint8 and vec_a_add.dtype == torch.int32 and vec_b_add.dtype == torch.int32
+    assert vec_a_mul.dtype in _FLOAT16S and vec_b_mul.dtype == vec_a_mul.dtype and out.dtype == vec_a_mul.dtype
+    assert mat_a.is_contiguous() and mat_b.is_contiguous() and vec_a_add.is_contiguous() and vec_b_add.is_contiguous() and vec_a_mul.is_contiguous() and vec_b_mul.is_contiguous() and out.is_contiguous()
+    assert mat_a.size(1) == mat_b.size(1) and vec_a_add.numel() == m and vec_a_mul.numel() == m
+    assert vec_b_add.numel() == n and vec_b_mul.numel() == n and out.shape == (m, n)
+    dev = require_gpu(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul, out)
+    with torch.cuda.device(dev):
+        rc = _lib.load().quest_fused_matmul_dequantize_add_int4_int4t(
+            ptr(out), ptr(mat_a), ptr(mat_b), ptr(vec_a_add), ptr(vec_b_add), ptr(vec_a_mul), ptr(vec_b_mul),
+            m, mat_b.size(1) * 2, n, DTYPE_CODE[out.dtype], stream_of(out))
+    if rc == QUEST_ERR_UNSUPPORTED:                                  # nothing was launched: the two calls
+        out += fused_matmul_dequantize_int4_int4t_bf16(mat_a, mat_b, vec_a_add, vec_b_add, vec_a_mul, vec_b_mul)
+        return out
+    check(rc, 'fused_matmul_dequantize_add_int4_int4t')
     return out
 
 

@@ -140,10 +140,13 @@ def main():
     ap.add_argument('--markdown', help='write the table to this file')
     ap.add_argument('--min-k', type=int, default=None, help='shortest rows that take the FP6 path (default: harness.E2M3_MIN_K)')
     ap.add_argument('--no-gemm-add', action='store_true', help='residual additions in the norm kernels instead of the output projections\' GEMMs')
+    ap.add_argument('--no-packed-gemm-add', action='store_true', help='no residual additions in the INT8 large-tile GEMM (the FP6 GEMM keeps its own)')
     ap.add_argument('--no-gemm-rope', action='store_true', help='rotary embedding in its own kernel instead of the QKV projection\'s GEMM')
     args = ap.parse_args()
     if args.no_gemm_add:
         harness.GEMM_ADDS_RESIDUAL = False
+    if args.no_packed_gemm_add:
+        harness.GEMM_ADDS_RESIDUAL_PACKED = False
     if args.no_gemm_rope:
         harness.GEMM_ROTATES_QK = False
     if args.min_k is not None:

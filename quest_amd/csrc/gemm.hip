@@ -62,9 +62,10 @@ static int small_tile_shape(int M, int K, int N, int cus) {
 // faster shape, and within 7 % on every single size.
 static int gemm_launch_large(int out_kind, bool glu, void *out, const uint8_t *a, const uint8_t *b, const int32_t *a_add,
                              const int32_t *b_add, const void *a_mul, const void *b_mul, int M, int K, int N, int cus,
-                             hipStream_t st, const RopeArgs *rope = nullptr) {
+                             hipStream_t st, const RopeArgs *rope = nullptr, bool add = false) {
     const int small_shape = small_tile_shape(M, K, N, cus);
-    const int epi = rope != nullptr ? kEpiRope : glu ? kEpiGlu : kEpiPlain;
+    const int epi = add ? kEpiAdd : rope != nullptr ? kEpiRope : glu ? kEpiGlu : kEpiPlain;
+    if (small_shape != 0 && add) return QUEST_ERR_UNSUPPORTED;           // the small tiles do not add into their output
     if (small_shape != 0) return launch_gemm_small(out_kind, epi, small_shape, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, st, rope);
     const int units = (N + 31) / 32;
     const int per_group = units >= 8 ? units / 8 : units;
@@ -221,6 +222,34 @@ extern "C" int quest_fused_matmul_dequantize_rope_int4_int4t(void *mat_d, const 
     return gemm_launch_large(dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16, false, mat_d, mat_a, mat_b, vec_a_add, vec_b_add,
                              vec_a_mul, vec_b_mul, size_m, size_k, size_n, device_cu_count((hipStream_t)stream),
                              (hipStream_t)stream, &rope);
+}
+
+// Whether quest_fused_matmul_dequantize_add_int4_int4t runs this size in one launch (the large-tile kernel takes it)
+static bool add_gemm_applies(int M, int K, int N, int cus) {
+    return (K & 127) == 0 && M > 64 && !(M <= 128 && N <= 8192) && small_tile_shape(M, K, N, cus) == 0;
+}
+
+extern "C" int quest_fused_matmul_dequantize_add_available(int size_m, int size_k, int size_n, void *stream) {
+    forget_stale_error();
+    if (size_m <= 0 || size_k <= 0 || size_n <= 0) return 0;
+    return add_gemm_applies(size_m, size_k, size_n, device_cu_count((hipStream_t)stream)) ? 1 : 0;
+}
+
+extern "C" int quest_fused_matmul_dequantize_add_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,
+                                                            const int32_t *vec_a_add, const int32_t *vec_b_add,
+                                                            const void *vec_a_mul, const void *vec_b_mul, int size_m,
+                                                            int size_k, int size_n, int dtype, void *stream) {
+    forget_stale_error();
+    const int rc = gemm_check(mat_d, mat_a, mat_b, size_m, size_k, size_n);
+    if (rc != QUEST_OK) return rc;
+    if (!vec_a_add || !vec_b_add || !vec_a_mul || !vec_b_mul) return QUEST_ERR_NULL_POINTER;
+    if (!check_dtype(dtype)) return QUEST_ERR_BAD_DTYPE;
+    const int cus = device_cu_count((hipStream_t)stream);
+    // only the large-tile kernel has this epilogue
+    if (!add_gemm_applies(size_m, size_k, size_n, cus) || !aligned(vec_b_mul, 4) || !aligned(vec_a_mul, 4) || !aligned(mat_d, 16))
+        return QUEST_ERR_UNSUPPORTED;
+    return gemm_launch_large(dtype == QUEST_DTYPE_BF16 ? OUT_BF16 : OUT_FP16, false, mat_d, mat_a, mat_b, vec_a_add, vec_b_add,
+                             vec_a_mul, vec_b_mul, size_m, size_k, size_n, cus, (hipStream_t)stream, nullptr, true);
 }
 
 extern "C" int quest_fused_matmul_dequantize_swiglu_int4_int4t(void *mat_d, const uint8_t *mat_a, const uint8_t *mat_b,

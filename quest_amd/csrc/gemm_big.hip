@@ -184,6 +184,7 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
     constexpr int DT = OUT == OUT_INT32 ? 0 : OUT;
     constexpr bool GLU = EPI == kEpiGlu;
     constexpr bool ROPE = EPI == kEpiRope;
+    constexpr bool ADD = EPI == kEpiAdd;
     static_assert(EPI == kEpiPlain || OUT != OUT_INT32, "epilogues on 16-bit outputs only");
     constexpr int NAX = NA > 0 ? NA : 1;
     // Lane coordinates are derived afresh in every phase (here, in the loader's cursor step, in the epilogue): a value
@@ -365,6 +366,16 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
             rope_fetch(rope, rl, lg_e, kTokOuter ? i : o, kTokOuter ? o : i, piece & 1, cs[par]);
         };
         if constexpr (ROPE) fetch_angles(0, 0);
+        // kEpiAdd: what the output holds under this lane's sixteen-byte pieces, fetched one piece ahead as well
+        uint4 res[2];
+        auto fetch_res = [&](int piece, int par) {
+            const int o = piece / (2 * kInner), i = (piece >> 1) % kInner, pr = piece & 1;
+            const int a = kTokOuter ? i : o, b = kTokOuter ? o : i;
+            const bool ok = !kGuard || (tok0 + tok_e + b * 32 + li_e < M && ch0 + (unit0 + a) * 32 + (2 * pr + lg_e) * 8 < N);
+            res[par] = make_uint4(0, 0, 0, 0);
+            if (ok) res[par] = *reinterpret_cast<const uint4 *>(out_lane + ((size_t)b * 32 * n_out + a * kOutPerUnit) * kEs + (2 * pr + lg_e) * 16);
+        };
+        if constexpr (ADD) fetch_res(0, 0);
 #pragma unroll
         for (int o = 0; o < kOuter; o++) {
 #pragma unroll
@@ -408,10 +419,14 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                         const auto s0 = __builtin_amdgcn_permlane32_swap(x[2 * pr][0], x[2 * pr + 1][0], false, false);
                         const auto s1 = __builtin_amdgcn_permlane32_swap(x[2 * pr][1], x[2 * pr + 1][1], false, false);
                         const int cl = (unit0 + a) * 32 + (2 * pr + lg_e) * 8;
-                        if constexpr (ROPE) {
+                        if constexpr (ROPE || ADD) {
                             constexpr int kPieces = 2 * kOuter * kInner;
                             const int nxt = (o * kInner + i) * 2 + pr + 1;
-                            if (nxt < kPieces) fetch_angles(nxt, (pr + 1) & 1);
+                            if constexpr (ROPE) {
+                                if (nxt < kPieces) fetch_angles(nxt, (pr + 1) & 1);
+                            } else {
+                                if (nxt < kPieces) fetch_res(nxt, (pr + 1) & 1);
+                            }
                         }
                         if constexpr (GLU) {
                             // The weight rows come interleaved in eights, four gate rows then the four up rows of the same
@@ -424,6 +439,13 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                             uint4 piece = make_uint4(s0[0], s1[0], s0[1], s1[1]);
                             if constexpr (ROPE) {
                                 if (ch0 + cl < rope.rot_cols) piece = rope_turn<DT>(piece, cs[pr]);
+                            }
+                            if constexpr (ADD) {                  // dtype(out + dtype(product)): the residual stream's addition
+                                const uint4 r = res[pr];
+                                auto add2 = [](uint32_t p, uint32_t q) {
+                                    return pack2_rounded_products<DT>(__fadd_rn(lo_f32<DT>(q), lo_f32<DT>(p)), __fadd_rn(hi_f32<DT>(q), hi_f32<DT>(p)));
+                                };
+                                piece = make_uint4(add2(piece.x, r.x), add2(piece.y, r.y), add2(piece.z, r.z), add2(piece.w, r.w));
                             }
                             *reinterpret_cast<uint4 *>(dst + (2 * pr + lg_e) * 16) = piece;
                         }
@@ -462,7 +484,13 @@ __device__ __forceinline__ void big_tile(uint8_t *lds, Cursor &ld, Loader &ldr, 
                         } else {
                             const float lhs = (float)(c * 2 + t_add + v_add[cl + e]);
                             const float rhs = __fmul_rn(t_half_mul, to_f32<DT>(v_mul[cl + e]));
-                            reinterpret_cast<uint16_t *>(out)[o] = (uint16_t)from_f32<DT>(__fmul_rn(lhs, rhs));
+                            uint32_t val = from_f32<DT>(__fmul_rn(lhs, rhs));
+                            if constexpr (ADD) {
+                                float sum = __fadd_rn(to_f32<DT>(reinterpret_cast<uint16_t *>(out)[o]), to_f32<DT>((uint16_t)val));
+                                asm volatile("" : "+v"(sum));
+                                val = from_f32<DT>(sum);
+                            }
+                            reinterpret_cast<uint16_t *>(out)[o] = (uint16_t)val;
                         }
                     }
                 }
@@ -596,6 +624,7 @@ int launch_gemm_big(int out_kind, int epi, bool duo, void *out, const uint8_t *a
                           : launch_shape<OUT_FP16, E>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope))
     if (epi == kEpiGlu) return QUEST_BIG_EPI(kEpiGlu);
     if (epi == kEpiRope) return QUEST_BIG_EPI(kEpiRope);
+    if (epi == kEpiAdd) return QUEST_BIG_EPI(kEpiAdd);
     if (epi != kEpiPlain) return QUEST_ERR_UNSUPPORTED;
     if (out_kind == OUT_INT32) return launch_shape<OUT_INT32, kEpiPlain>(duo, out, a, b, a_add, b_add, a_mul, b_mul, M, K, N, cus, st, rope);
     return QUEST_BIG_EPI(kEpiPlain);

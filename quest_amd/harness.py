@@ -26,6 +26,7 @@ E2M3_MIN_K = 2048                       # shortest rows that take it (see prefer
 # Whether a producer-fused block lets the FP6 GEMM of an output projection add into the residual stream itself
 # (same bits as the addition inside the next norm kernel; one pass over the stream less).
 GEMM_ADDS_RESIDUAL = True
+GEMM_ADDS_RESIDUAL_PACKED = True       # ... also on packed nibbles, where the INT8 large-tile kernel takes the projection
 # ... and the rotary embedding of q and k after the fused QKV projection (the FP6 GEMM's rotary epilogue)
 GEMM_ROTATES_QK = True
 
@@ -243,13 +244,19 @@ class Linear4bit(nn.Module):
         self.bias = nn.Parameter(torch.zeros(out_features, dtype=dtype, device=device), requires_grad=False) if bias else None
         return self
 
-    def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None, rope=None) -> torch.Tensor:
+    def forward_quantized(self, a_scale, a_int_packed, a_int_row_sum, out=None, rope=None, add_to_out=False) -> torch.Tensor:
         """The GEMM half of `linear_forward` on activations some fused producer kernel has already quantised:
         (M, 1) scales, (M, K/2) codes, (M, 1) row sums -> (M, N).  In no-op mode the GEMM is skipped (zeros), which is
         what prices the GEMMs of a producer-fused model: everything else, the quantising producers included, still runs.
-        rope = (freqs_cis, rot_cols, head_dim): the first rot_cols channels leave rotated (layers without a bias)."""
+        rope = (freqs_cis, rot_cols, head_dim): the first rot_cols channels leave rotated (layers without a bias).
+        add_to_out: the result is added to `out` (the residual stream), with the bits of `out + layer(x)` (layers without
+        a bias; one launch where `quest.gemm_add_fuses` says so)."""
         if self.use_noop:
-            return self._noop_output(a_scale)
+            return out if add_to_out else self._noop_output(a_scale)
+        if add_to_out:
+            assert self.bias is None and rope is None and out is not None
+            return quest.fused_matmul_dequantize_add_int4_int4t(a_int_packed, self.w_int_packed, a_int_row_sum, self.w_add,
+                                                                a_scale, self.w_scale, out)
         if rope is not None:
             assert self.bias is None
             return quest.fused_matmul_dequantize_rope_int4_int4t(a_int_packed, self.w_int_packed, a_int_row_sum, self.w_add,

@@ -244,9 +244,16 @@ class LlamaBlock(nn.Module):
         # x + c_proj(...)) and the second norm has no addition left to do; otherwise the norm kernel adds
         att = None
         gemm_adds = harness.GEMM_ADDS_RESIDUAL
-        if gemm_adds and harness.prefers_e2m3(m, c, c) and isinstance(self.attn.c_proj, harness.Linear4bit) and self.attn.c_proj.use_hadamard:
+        o_proj = self.attn.c_proj
+        packed_adds = (isinstance(o_proj, harness.Linear4bit) and o_proj.use_hadamard and o_proj.bias is None
+                       and not o_proj.quantize_from_fp32)
+        if gemm_adds and harness.prefers_e2m3(m, c, c) and isinstance(o_proj, harness.Linear4bit) and o_proj.use_hadamard:
             core = self.attn.attention_core(qkv.view(b, t, 3 * c), freqs_cis, rotated)
-            self.attn.c_proj.forward_tiles(*quest.hadamard_quantize_e2m3(core.view(m, c)), out=x2, add_to_out=True)
+            o_proj.forward_tiles(*quest.hadamard_quantize_e2m3(core.view(m, c)), out=x2, add_to_out=True)
+        elif gemm_adds and harness.GEMM_ADDS_RESIDUAL_PACKED and packed_adds and quest.gemm_add_fuses(m, c, c, x.device):
+            # the same on packed nibbles where the INT8 large-tile kernel takes the projection
+            core = self.attn.attention_core(qkv.view(b, t, 3 * c), freqs_cis, rotated)
+            o_proj.forward_quantized(*quest.hadamard_quantize_int4(core.view(m, c)), out=x2, add_to_out=True)
         else:
             att = self.attn.attend(qkv.view(b, t, 3 * c), freqs_cis, rotated)
         down_tiles = harness.prefers_e2m3(m, hidden, c)
@@ -277,6 +284,11 @@ class LlamaBlock(nn.Module):
         if down_tiles and gemm_adds:
             # the MLP's output projection adds into the residual stream as well: nothing is left for the caller to add
             self.mlp.c_proj.forward_tiles(*q, out=x2, add_to_out=True)
+            return x, None
+        down = self.mlp.c_proj
+        if (not down_tiles and gemm_adds and harness.GEMM_ADDS_RESIDUAL_PACKED and isinstance(down, harness.Linear4bit) and down.use_hadamard and down.bias is None
+                and not down.quantize_from_fp32 and quest.gemm_add_fuses(m, hidden, c, x.device)):
+            down.forward_quantized(*q, out=x2, add_to_out=True)
             return x, None
         y = self.mlp.c_proj.forward_tiles(*q) if down_tiles else self.mlp.c_proj.forward_quantized(*q)
         return x, y.view(b, t, c)

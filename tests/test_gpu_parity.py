@@ -274,6 +274,44 @@ def test_swiglu_gemm_refuses_small_batches(quest):
                                                         torch.ones(n, 1, dtype=torch.bfloat16, device=DEV))
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(300, 384, 1000), (16384, 128, 1024), (4096, 1024, 3072), (165, 128, 392), (256, 128, 64),
+                                   (1000, 128, 4100), (2048, 2560, 2560), (4099, 128, 1031), (48, 256, 128), (256, 256, 192),
+                                   (80, 160, 64)])
+def test_fused_matmul_dequantize_adds_into_the_residual_stream(quest, dtype, shape):
+    """out <- dtype(out + dtype(product)) on packed codes: the bits of torch's `out + product`, in the large-tile kernel's
+    epilogue (both its shapes, narrow tiles, edge tiles, a channel count that is not a multiple of 8, large and tiny
+    residuals, twice on one buffer) and as two launches where another kernel takes the size -- which
+    `gemm_add_fuses` tells beforehand."""
+    m, k, n = shape
+    g = torch.Generator().manual_seed(47)
+    a, b = rand_codes(m, k, 48).to(DEV), rand_codes(n, k, 49).to(DEV)
+    a_mul = (torch.rand(m, 1, generator=g) * 0.05 + 0.01).to(dtype).to(DEV)
+    b_mul = (torch.rand(n, 1, generator=g) * 0.05 + 0.01).to(dtype).to(DEV)
+    a_add = torch.randint(-200, 200, (m, 1), generator=g, dtype=torch.int32).to(DEV)
+    b_add = torch.randint(-200, 200, (n, 1), generator=g, dtype=torch.int32).to(DEV)
+    product = quest.fused_matmul_dequantize_int4_int4t_bf16(a, b, a_add, b_add, a_mul, b_mul)
+    res = (torch.randn(m, n, generator=g) * torch.rand(m, 1, generator=g) * 50).to(dtype)
+    res[0] *= 1e-4
+    res = res.to(DEV)
+    want = res + product
+    got = res.clone()
+    ret = quest.fused_matmul_dequantize_add_int4_int4t(a, b, a_add, b_add, a_mul, b_mul, got)
+    assert ret.data_ptr() == got.data_ptr()
+    assert torch.equal(bits(got.cpu()), bits(want.cpu()))
+    quest.fused_matmul_dequantize_add_int4_int4t(a, b, a_add, b_add, a_mul, b_mul, got)
+    assert torch.equal(bits(got.cpu()), bits((want + product).cpu()))
+    from quest_amd import _lib
+    rc = _lib.load().quest_fused_matmul_dequantize_add_int4_int4t(
+        got.data_ptr(), a.data_ptr(), b.data_ptr(), a_add.data_ptr(), b_add.data_ptr(), a_mul.data_ptr(), b_mul.data_ptr(),
+        m, k, n, 0 if dtype == torch.bfloat16 else 1, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert (rc == 0) == quest.gemm_add_fuses(m, k, n) and rc in (0, -5)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    small = k % 256 == 0 and (-(-(-(-m // 64) * -(-n // 64)) // cus) <= 4 or (-(-(-(-m // 64) * -(-n // 64)) // cus) <= 8 and m < 1024 and m % 256))
+    assert quest.gemm_add_fuses(m, k, n) == (_tiled_kernel_takes(m, k, n) and not small)
+
+
 def _tiled_kernel_takes(m, k, n):
     """The dispatch of the fused GEMM (gemm.hip), restated: whether the large-tile or the small-tile kernel gets this size
     (the two with the rotary epilogue) rather than the weight-streaming or the register-staged one."""
