@@ -49,8 +49,8 @@ FP6_MFMA_PEAK_TOPS = 10100.0
 # the runs are summarised under profiles/.
 TRAFFIC_SOURCE = ('constant from a separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this script, summarised in '
                   'profiles/bench_gemm_e2m3_M4096_K4096_N11008_and_quantize_8192x4096.md; not measured in this run')
-TRAFFIC_GEMM_BYTES = 337035025                 # gemm_e2m3_kernel; of these 227.2 MB fetched (operands: 46.4 MB), 109.9 MB written
-TRAFFIC_QUANTIZE_BYTES = 84284027
+TRAFFIC_GEMM_BYTES = 329496400                 # gemm_e2m3_kernel; of these 219.7 MB fetched (operands: 46.4 MB), 109.8 MB written
+TRAFFIC_QUANTIZE_BYTES = 84284627
 # what quest_e2m3_gemm_plan reported for M=4096 K=4096 N=11008 on 256 compute units when TRAFFIC_GEMM_BYTES was measured: the
 # figure depends on the schedule (which workgroup fetches what), so the line says `traffic_stale` when the plan has changed
 TRAFFIC_GEMM_PLAN = [256, 8, 0, 2, 256, 256, 6, 64]
