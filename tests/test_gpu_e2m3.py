@@ -215,6 +215,49 @@ def test_gemm_rotates_q_and_k(quest, dtype, shape):
     assert not torch.equal(bits(got[:, :2 * c].cpu()), bits(plain[:, :2 * c].cpu()))
 
 
+@pytest.mark.parametrize('seed', range(16))
+def test_epilogues_seeded_fuzz(quest, seed):
+    """Random shapes: the rotary and the residual-add epilogues of the FP6 GEMM and of the packed-nibble GEMM (whichever
+    kernel takes the size) against the plain packed-nibble GEMM followed by the rotary kernel / by torch's addition."""
+    import random
+    rnd = random.Random(5000 + seed)
+    dtype = DTYPES[seed % 2]
+    hd = rnd.choice([32, 64, 96, 128])
+    heads = rnd.randint(1, 12)
+    c = heads * hd
+    n = 2 * c + 8 * rnd.randint(0, 40)
+    t = rnd.choice([32, 33, 64, 100, 128, 512])
+    bsz = rnd.choice([1, 2, 3, 5, 8, rnd.randint(1, 16)])
+    m, k = bsz * t, 128 * rnd.randint(1, 24)
+    g = torch.Generator(device=DEV).manual_seed(6000 + seed)
+    a = torch.randint(0, 256, (m, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    b = torch.randint(0, 256, (n, k // 2), generator=g, device=DEV, dtype=torch.uint8)
+    a_mul = (torch.rand(m, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    b_mul = (torch.rand(n, 1, generator=g, device=DEV) * 0.09 + 0.01).to(dtype)
+    from quest_amd import harness
+    a_add = harness.unpack_int4(a).to(torch.int32).sum(-1, keepdim=True).to(torch.int32)
+    b_add = harness.unpack_int4(b).to(torch.int32).sum(-1, keepdim=True).to(torch.int32) + k // 2
+    ang = torch.rand(t, hd // 2, generator=g, device=DEV) * 6.283
+    freqs = torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).contiguous()
+    plain = quest.fused_matmul_dequantize_int4_int4t_bf16(a, b, a_add, b_add, a_mul, b_mul)
+    want = plain.clone()
+    quest.rope_interleaved_(want.view(bsz, t, n), freqs, 2 * c, hd)
+    case = (m, t, k, n, heads, hd)
+    got = quest.fused_matmul_dequantize_rope_int4_int4t(a, b, a_add, b_add, a_mul, b_mul, freqs, 2 * c, hd)
+    assert torch.equal(bits(got.cpu()), bits(want.cpu())), case
+    ta, tb = quest.int4_to_e2m3_tiles(a), quest.int4_to_e2m3_tiles(b)
+    got = quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k, rope=(freqs, 2 * c, hd))
+    assert torch.equal(bits(got.cpu()), bits(want.cpu())), case
+    res = (torch.randn(m, n, generator=g, device=DEV) * 30).to(dtype)
+    want = res + plain
+    got = res.clone()
+    quest.fused_matmul_dequantize_add_int4_int4t(a, b, a_add, b_add, a_mul, b_mul, got)
+    assert torch.equal(bits(got.cpu()), bits(want.cpu())), case
+    got = res.clone()
+    quest.fused_matmul_dequantize_e2m3(ta, tb, a_mul, b_mul, k, out=got, add_to_out=True)
+    assert torch.equal(bits(got.cpu()), bits(want.cpu())), case
+
+
 def test_rope_epilogue_rejects_what_it_does_not_take(quest):
     from quest_amd import _lib
     import ctypes
